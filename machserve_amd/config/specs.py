@@ -26,6 +26,10 @@ class NormSpec:
     width: int
     eps: float
     tensors: Mapping[str, str] = field(default_factory=dict)
+    # a norm whose weight is stored around zero: the weight applied is ``offset`` plus the stored one
+    offset: float = 0.0
+    # whether a second vector ("scale" among the tensors) multiplies the normed row as well (a layer's scale)
+    scaled: bool = False
 
 
 @dataclass(frozen=True)
@@ -189,13 +193,102 @@ class LightningSpec:
 
 
 @dataclass(frozen=True)
+class ChunkedAttentionSpec:
+    """Grouped-query attention with keys ``head_dim`` and values ``v_head_dim`` wide, behind a short convolution on q, k and v.
+
+    ``q, k, v = W h (+ bias)``; with ``conv_taps`` > 0 a causal convolution over time on every channel of q, k and v
+    (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, no bias), whose last ``conv_taps - 1`` inputs are a request's state; with
+    ``qk_norm`` an RMS norm (``norm_eps``, a weight per coordinate) over the whole of q and one over the whole of k;
+    ``position``: the rotation of q and k (its ``rotary_dim`` first numbers of a head, pairs as its ``pairing`` says; None:
+    none); ``score = scale q . k``, then with ``softcap`` ``softcap tanh(score / softcap)``; a row at position i sees the
+    keys j <= i with ``floor(i / chunk) = floor(j / chunk)`` (``chunk`` None: every j <= i) and, with ``window``, ``i - j <
+    window``; softmax; output projection."""
+    kind: str
+    hidden: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    position: Optional[RotarySpec] = None
+    conv_taps: int = 0
+    bias: bool = True
+    qk_norm: bool = True
+    norm_eps: float = 1e-6
+    softcap: float = 0.0
+    chunk: Optional[int] = None
+    window: Optional[int] = None
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class GatedRecurrenceSpec:
+    """A recurrent block around a real-gated linear recurrent unit: two branches of ``width`` channels,
+    ``y = gelu_tanh(W_y h + b_y)`` and ``u = conv(W_x h + b_x) + b_conv`` (a causal convolution of ``conv_taps`` taps per
+    channel); the channels are cut into ``blocks`` equal parts, in each ``r = sigmoid(A u + b_a)`` and ``i = sigmoid(B u +
+    b_i)`` with square matrices; ``a = exp(-decay_factor r softplus(lam))``, ``S <- a S + sqrt(1 - a^2) (i u)`` from zero;
+    the output is ``W_o (S y)``."""
+    kind: str
+    hidden: int
+    width: int
+    blocks: int
+    conv_taps: int
+    decay_factor: float = 8.0
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class TimeMixSpec:
+    """Time mixing with a decay per key channel that depends on the token.  Each of r, k, v, g, w reads its own mix of a
+    token's input with the one before it, ``h + (h' - h) mu``; ``r, k, v = W mix`` (``heads`` x ``head_dim``), the gate
+    ``silu(W_g mix_g)``, the decay ``w = exp(-exp(W_2 tanh(W_1 mix_w) + w0))`` through a bottleneck of ``decay_rank`` (None:
+    whatever the checkpoint's tensors have); per head ``o = (S + diag(u) k v^T)^T r``, ``S <- diag(w) S + k v^T``; a head's
+    ``o`` is divided by its root mean square (``norm_eps``), times a weight, times the gate, and projected."""
+    kind: str
+    hidden: int
+    heads: int
+    head_dim: int
+    decay_rank: Optional[int] = None
+    norm_eps: float = 1e-6
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Several mixers that read the same input; each one's output is RMS-normed over the model's width (``norm_eps``) with a
+    weight of its own (``tensors``: ``norm.<i>``), and the result is their mean."""
+    kind: str
+    hidden: int
+    branches: Sequence[object]
+    norm_eps: float = 1e-6
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class RoutedMlpSpec:
+    """A feed-forward of ``experts`` small layers ``W_down act(W_up h)`` without biases, of which a token uses the ``top``
+    with the largest router logits ``W_r h (+ bias)``, weighted by the softmax over the chosen logits alone; with
+    ``shared`` > 0 one more such layer of that size runs for every token and is added."""
+    kind: str
+    hidden: int
+    experts: int
+    top: int
+    intermediate: int
+    activation: str = "gelu"
+    shared: int = 0
+    router_bias: bool = True
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
 class GatedMlpSpec:
-    """``down(act(gate(x)) * up(x))``."""
+    """``down(act(gate(x)) * up(x))``; with ``bias`` every projection has one."""
     kind: str
     hidden: int
     intermediate: int
     activation: str = "silu"
     tensors: Mapping[str, str] = field(default_factory=dict)
+    bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -224,6 +317,17 @@ class SandwichLayerSpec:
 
 
 @dataclass(frozen=True)
+class PostNormLayerSpec:
+    """A block whose branches read the stream itself and are normed on their way out: ``x += post(mixer(x))``, then
+    ``x += post(feed_forward(x))``; ``feed_forward`` None: the layer has none."""
+    block: str
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_post_norm: object
+    feed_forward_post_norm: Optional[object]
+
+
+@dataclass(frozen=True)
 class ParallelLayerSpec:
     """A block whose branches read one norm: ``h = norm(x); x += mixer(h) + feed_forward(h)``; ``feed_forward`` None:
     the layer has none."""
@@ -241,6 +345,19 @@ class EmbeddingSpec:
     tensors: Mapping[str, str] = field(default_factory=dict)
     kind: str = "embedding"
     scale: float = 1.0
+
+
+@dataclass(frozen=True)
+class PairEmbeddingSpec:
+    """Token embedding plus a row of a second table chosen by the token and the one before it: row ``(previous * mul_prev +
+    token * mul_cur) mod buckets``, and row ``buckets`` (the last) for a request's first token."""
+    vocab: int
+    width: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    tensors: Mapping[str, str] = field(default_factory=dict)
+    kind: str = "pair_embedding"
 
 
 @dataclass(frozen=True)

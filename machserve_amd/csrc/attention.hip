@@ -89,7 +89,24 @@ struct AttnArgs {
     const float* sinks;
     // [T, H] or null: what the output of (row, head) is multiplied by (a gate), in the same pass as the softmax's division
     const float* out_gate;
+    // chunk > 0: a row at position p sees only the keys from floor(p / chunk) * chunk on (chunks counted from the
+    // request's position 0), beside whatever the window leaves
+    int chunk;
+    // softcap > 0: the scaled score s becomes softcap * tanh(s / softcap) before the softmax
+    float softcap;
 };
+
+// The first key a row at `pos` sees under a window and a chunked mask (either 0: none).
+__device__ __forceinline__ int first_visible_key(int pos, int window, int chunk) {
+    int lo = window > 0 ? pos - window + 1 : 0;
+    if (chunk > 0) lo = max(lo, pos / chunk * chunk);
+    return lo;
+}
+
+// A raw score under the cap, still in the units that the softmax's scale multiplies: scale * result = cap * tanh(scale * s / cap).
+__device__ __forceinline__ float capped_raw(float s, float scale, float softcap) {
+    return softcap / scale * tanhf(s * (scale / softcap));
+}
 
 __device__ __forceinline__ float exp_f(float x) {
 #ifdef MS_ELEM_HALF
@@ -176,8 +193,8 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     const int last_row = min(r0 + 64, R) - 1;
     int kv_hi = pos0 + last_row / g + 1;
     int kv_lo = 0;
-    if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
-    const int lo_key = a.window > 0 ? pos - a.window + 1 : 0;
+    if (a.window > 0 || a.chunk > 0) kv_lo = max(0, first_visible_key(pos0 + r0 / g, a.window, a.chunk));
+    const int lo_key = first_visible_key(pos, a.window, a.chunk);
     const int sp = blockIdx.y;
     if (a.nsplit > 1) {
         const int first = (kv_lo / ROUND) * ROUND;
@@ -345,7 +362,7 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     // rows of this wave: the first and the last position decide which tiles need no mask at all
     const int pos_first = pos0 + (r0 + wave * 16) / g;
     const int pos_last = pos0 + min(r0 + wave * 16 + 15, max(R - 1, 0)) / g;
-    const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
+    const int lo_last = first_visible_key(pos_last, a.window, a.chunk);
 
     // Round r: group kg has the tile of absolute index round_first * KG + r * KG + kg.  Its loads are
     // asked for PF rounds ahead into register slot r % PF, it is written into LDS stage r % 2 while
@@ -396,6 +413,12 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
             ahead = lookup();
         }
         if (busy) {
+        if (a.softcap > 0.f) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[nt][i] = capped_raw(sc[nt][i], a.scale, a.softcap);
+        }
         // a tile that every row of the wave sees whole needs no mask
         const bool whole = kt0 + BKV - 1 <= pos_first && kt0 >= lo_last;
         float tmax = NEG_BIG;
@@ -616,8 +639,8 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     const int last_row = min(r0 + ROWS_PER_BLOCK, R) - 1;
     int kv_hi = pos0 + last_row / g + 1;
     int kv_lo = 0;
-    if (a.window > 0) kv_lo = max(0, pos0 + r0 / g - a.window + 1);
-    const int lo_key = a.window > 0 ? pos - a.window + 1 : 0;
+    if (a.window > 0 || a.chunk > 0) kv_lo = max(0, first_visible_key(pos0 + r0 / g, a.window, a.chunk));
+    const int lo_key = first_visible_key(pos, a.window, a.chunk);
     const int sp = blockIdx.y;
     if (a.nsplit > 1) {
         const int first = (kv_lo / ROUND) * ROUND;
@@ -718,7 +741,7 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     // rows of this wave: the first and the last position decide which tiles need no mask at all
     const int pos_first = pos0 + (r0 + rw * 32) / g;
     const int pos_last = pos0 + min(r0 + rw * 32 + 31, max(R - 1, 0)) / g;
-    const int lo_last = a.window > 0 ? pos_last - a.window + 1 : 0;
+    const int lo_last = first_visible_key(pos_last, a.window, a.chunk);
     // where this lane reads its fragments in a stage: row n32 of the K tile, row 32 dt + n32 of V^T, chunk 2c + h
     const int k_row = n32 * (HDT * 2), k_sw = k_swizzle(n32), v_row = K_BYTES + n32 * (TK * 2), v_sw = v_swizzle(n32);
 
@@ -780,6 +803,10 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
             Frag vf[NDT];
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) vf[dt] = v_frag(0, dt);
+            if (a.softcap > 0.f) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sc[i] = capped_raw(sc[i], a.scale, a.softcap);
+            }
             const bool whole = kt0 + TK - 1 <= pos_first && kt0 >= lo_last;
             if (!whole) {
 #pragma unroll
@@ -906,6 +933,8 @@ struct DecodeArgs {
     int n_partials, stride;
     const float* sinks;      // [H] or null: see AttnArgs
     const float* out_gate;   // [S, H] or null: see AttnArgs
+    int chunk;               // see AttnArgs
+    float softcap;           // see AttnArgs
 };
 
 constexpr int MAX_SPLITS = 64;
@@ -938,7 +967,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     // keys read from the pages: all of them, or (fused) those before the row's own position,
     // whose key and value are still in registers and enter as one extra term
     const int kv_len = FUSED ? pos : pos + 1;
-    const int lo_key = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const int lo_key = max(0, first_visible_key(pos, a.window, a.chunk));
     const int* table = a.block_table + (size_t)s * a.table_stride;
     const bool valid = r16 < g;
     const int head = kvh * g + (valid ? r16 : 0);
@@ -1180,7 +1209,9 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
             for (int i = 0; i < 4; ++i) {
                 const int key = kt0 + score_key(nt, i);
                 const bool ok = valid && key < kv_len && key >= lo_key;
-                const float v = ok ? sc[nt][i] * a.scale : -INFINITY;
+                float sv = sc[nt][i] * a.scale;
+                if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+                const float v = ok ? sv : -INFINITY;
                 sc[nt][i] = v;
                 tmax = fmaxf(tmax, v);
             }
@@ -1435,12 +1466,16 @@ extern "C" int MS_CAT(ms_attention_splits_nd, MS_ATTN_ND)(int n_work, int KV, in
 
 // `sinks`: null, or one number per head that the softmax's denominator also holds as exp(sink); `out_gate`: null, or
 // float [T, H] that the output of each (row, head) is multiplied by.
-extern "C" int MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(
+// `chunk`, `softcap`: see AttnArgs (0: none).  What a row can reach back (`reach`: the window, the chunk, or the smaller of
+// both) is what the choice of the kernel and of its key groups goes by.
+extern "C" int MS_CAT(ms_paged_attention_mask_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
-    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, int T, int nsplit, float* part_o,
-    float* part_ml, const float* sinks, const float* out_gate, hipStream_t stream) {
+    int hd, int ps, int n_pages, int window_of_mask, float scale, int max_key_groups, int T, int nsplit, float* part_o,
+    float* part_ml, const float* sinks, const float* out_gate, int chunk, float softcap, hipStream_t stream) {
     MS_REQUIRE(n_work > 0, "attention: no work");
+    MS_REQUIRE(chunk >= 0 && softcap >= 0.f && (softcap == 0.f || scale != 0.f), "attention: chunk %d, score cap %g", chunk, (double)softcap);
+    const int window = window_of_mask > 0 && chunk > 0 ? (window_of_mask < chunk ? window_of_mask : chunk) : (window_of_mask > 0 ? window_of_mask : chunk);
     MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml && T > 0)),
                "attention: %d key splits (at most %d, with their workspaces)", nsplit, MAX_SPLITS);
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "attention: head size %d does not fit this tile of %d", hd, HDT);
@@ -1449,7 +1484,8 @@ extern "C" int MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(
     MS_REQUIRE(window >= 0, "attention: window %d", window);
     MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
-               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0, nsplit, part_o, part_ml, sinks, out_gate};
+               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window_of_mask, scale, n_work, 0, nsplit, part_o, part_ml, sinks, out_gate,
+               chunk, softcap};
     // key groups per block by the longest context the block tables allow (the lengths themselves
     // are on the device): short contexts have no chain worth cutting
     const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
@@ -1509,6 +1545,16 @@ extern "C" int MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(
     return check_launch("attention_merge");
 }
 
+extern "C" int MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
+    const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
+    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, int T, int nsplit, float* part_o,
+    float* part_ml, const float* sinks, const float* out_gate, hipStream_t stream) {
+    return MS_CAT(ms_paged_attention_mask_nd, MS_ATTN_ND)(q, kpool, vpool, out, block_table, table_stride, seq_q_start, seq_q_len,
+                                                            seq_pos0, work, n_work, H, KV, hd, ps, n_pages, window, scale,
+                                                            max_key_groups, T, nsplit, part_o, part_ml, sinks, out_gate, 0, 0.f, stream);
+}
+
 extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
@@ -1524,22 +1570,32 @@ extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROW
 // Attention of a step in which every request has exactly one row (row s = request s).
 // part_o [S, H, nsplit, hd] and part_ml [S, H, nsplit, 2] are float workspaces (unused when
 // nsplit == 1).  Needs H / KV <= 16.
-extern "C" int MS_CAT(ms_decode_attention_ex_nd, MS_ATTN_ND)(
+extern "C" int MS_CAT(ms_decode_attention_mask_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
     int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
-    const float* sinks, const float* out_gate, hipStream_t stream) {
+    const float* sinks, const float* out_gate, int chunk, float softcap, hipStream_t stream) {
     MS_REQUIRE(S > 0, "decode attention: no rows");
+    MS_REQUIRE(chunk >= 0 && softcap >= 0.f, "decode attention: chunk %d, score cap %g", chunk, (double)softcap);
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "decode attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0 && H / KV <= 16, "decode attention: %d heads over %d key/value heads (at most 16 each)", H, KV);
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
     MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits (at most %d)", nsplit, MAX_SPLITS);
     DecodeArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table,
-                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0, sinks, out_gate};
+                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0, sinks, out_gate,
+                 chunk, softcap};
     hipLaunchKernelGGL(decode_attention_kernel<false>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
     int rc = check_launch("decode_attention");
     if (rc || nsplit == 1) return rc;
     hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit, a.sinks, H, a.out_gate);
     return check_launch("decode_merge");
+}
+
+extern "C" int MS_CAT(ms_decode_attention_ex_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
+    int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
+    const float* sinks, const float* out_gate, hipStream_t stream) {
+    return MS_CAT(ms_decode_attention_mask_nd, MS_ATTN_ND)(q, kpool, vpool, out, part_o, part_ml, block_table, table_stride, seq_pos0,
+                                                             S, H, KV, hd, ps, window, nsplit, scale, sinks, out_gate, 0, 0.f, stream);
 }
 
 extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(

@@ -317,6 +317,82 @@ __global__ __launch_bounds__(256) void conv_row_state_kernel(const float* __rest
     for (int i = 0; i < keep; ++i) st[(size_t)i * C + c] = v[i];
 }
 
+// ---- rows of q, k and v that are finished elsewhere (a convolution on all three, say), given as 32-bit numbers ------------
+// An RMS norm over the whole of q and one over the whole of k (weights; null: none), then the rotation of the first `rot`
+// numbers of every head of q and k by position * inv_freq, pairs (i, i + rot / 2) or neighbours (2i, 2i + 1); q goes out
+// in the element type with heads of dp numbers (zeros from d on), k and v into their pages, whose heads are dp wide too
+// (what lies beyond d, or beyond dv for a value, is never written and stays zero).
+struct FinishArgs {
+    const float* rows;      // [T, stride]: q [H, d], k [KV, d], v [KV, dv]
+    int stride;
+    const float* q_norm;    // [H * d] or null
+    const float* k_norm;    // [KV * d] or null
+    float eps;
+    const int* positions;   // [T]
+    const float* inv_freq;  // [rot / 2] or null: no rotation
+    int rot, neighbours;
+    const int* slot_map;    // [T] page * ps + offset
+    elem_t* q_out;          // [T, H * dp]
+    elem_t* kpool;          // [pages, KV, ps, dp]
+    elem_t* vpool;          // [pages, KV, dp, ps]
+    int H, KV, d, dv, dp, ps;
+};
+
+__global__ __launch_bounds__(256) void finish_rows_kernel(FinishArgs a) {
+    __shared__ float scratch[4];
+    extern __shared__ float lds[];
+    float* row = lds;                 // stride floats
+    float* cs = lds + a.stride;       // rot / 2 cosines, then rot / 2 sines
+    const int t = blockIdx.x, nq = a.H * a.d, nk = a.KV * a.d, nv = a.KV * a.dv, half = a.rot / 2;
+    float ssq = 0.f, ssk = 0.f;
+    for (int c = threadIdx.x; c < nq + nk + nv; c += 256) {
+        const float v = a.rows[(size_t)t * a.stride + c];
+        row[c] = v;
+        if (c < nq) ssq += v * v;
+        else if (c < nq + nk) ssk += v * v;
+    }
+    for (int j = threadIdx.x; j < half; j += 256) {
+        float c = 1.f, s = 0.f;
+        if (a.inv_freq) sincosf((float)a.positions[t] * a.inv_freq[j], &s, &c);
+        cs[j] = c;
+        cs[half + j] = s;
+    }
+    ssq = block_sum<256>(ssq, scratch);
+    ssk = block_sum<256>(ssk, scratch);
+    const float inv_q = a.q_norm ? 1.0f / sqrtf(ssq / (float)nq + a.eps) : 1.0f;
+    const float inv_k = a.k_norm ? 1.0f / sqrtf(ssk / (float)nk + a.eps) : 1.0f;
+    __syncthreads();
+    const int slot = a.slot_map[t];
+    const int page = slot >= 0 ? slot / a.ps : 0, off = slot >= 0 ? slot % a.ps : 0;
+    const int fill = a.dp - a.d;
+    for (int c = threadIdx.x; c < nq + nk; c += 256) {
+        const bool is_q = c < nq;
+        const int cc = is_q ? c : c - nq;
+        const int h = cc / a.d, i = cc - h * a.d;
+        const float inv = is_q ? inv_q : inv_k;
+        const float* nw = is_q ? a.q_norm : a.k_norm;
+        const float* base = row + (is_q ? 0 : nq) + h * a.d;
+        auto normed = [&](int e) { return base[e] * inv * (nw ? nw[h * a.d + e] : 1.0f); };
+        float v;
+        if (i >= a.rot) {
+            v = normed(i);
+        } else if (a.neighbours) {
+            const int pr = i >> 1;
+            v = (i & 1) ? normed(i) * cs[pr] + normed(i - 1) * cs[half + pr] : normed(i) * cs[pr] - normed(i + 1) * cs[half + pr];
+        } else {
+            v = i < half ? normed(i) * cs[i] - normed(i + half) * cs[half + i] : normed(i) * cs[i - half] + normed(i - half) * cs[i];
+        }
+        if (is_q) a.q_out[((size_t)t * a.H + h) * a.dp + i] = from_f32<elem_t>(v);
+        else if (slot >= 0) a.kpool[(((size_t)page * a.KV + h) * a.ps + off) * a.dp + i] = from_f32<elem_t>(v);
+    }
+    for (int c = threadIdx.x; c < a.H * fill; c += 256)  // the queries' heads are filled up with zeros
+        a.q_out[((size_t)t * a.H + c / fill) * a.dp + a.d + c % fill] = from_f32<elem_t>(0.f);
+    for (int c = threadIdx.x; c < nv; c += 256) {
+        const int h = c / a.dv, e = c - h * a.dv;
+        if (slot >= 0) a.vpool[(((size_t)page * a.KV + h) * a.dp + e) * a.ps + off] = from_f32<elem_t>(row[nq + nk + c]);
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -353,4 +429,18 @@ extern "C" int ms_conv_rows(const float* proj, int n_partials, int stride, const
     hipLaunchKernelGGL(conv_row_state_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, proj, n_partials, (size_t)T * stride, stride,
                        state, seq_q_start, seq_q_len, seq_slot, C, taps);
     return check_launch("conv_rows_state");
+}
+
+extern "C" int ms_finish_rows(const float* rows, int stride, const float* q_norm, const float* k_norm, float eps, const int* positions,
+                              const float* inv_freq, int rot, int neighbours, const int* slot_map, void* q_out, void* kpool, void* vpool,
+                              int T, int H, int KV, int d, int dv, int dp, int ps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && H > 0 && KV > 0 && d > 0 && dv > 0 && dp >= d && dp >= dv, "finish rows: %d rows, %d / %d heads of %d and %d in %d",
+               T, H, KV, d, dv, dp);
+    const int n = H * d + KV * d + KV * dv;
+    MS_REQUIRE(stride >= n && n + rot <= CONV_MAX_ROW, "finish rows: a row of %d numbers (stride %d, at most %d)", n, stride, CONV_MAX_ROW);
+    MS_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= d, "finish rows: %d of %d numbers of a head are rotated", rot, d);
+    FinishArgs a{rows, stride, q_norm, k_norm, eps, positions, inv_freq, rot, neighbours, slot_map, (elem_t*)q_out, (elem_t*)kpool,
+                 (elem_t*)vpool, H, KV, d, dv, dp, ps};
+    hipLaunchKernelGGL(finish_rows_kernel, dim3(T), dim3(256), (size_t)(stride + rot) * sizeof(float), stream, a);
+    return check_launch("finish_rows");
 }

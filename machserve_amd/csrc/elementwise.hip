@@ -192,8 +192,10 @@ __global__ __launch_bounds__(256) void add_partials_kernel(float* __restrict__ x
 
 // x[t, :] += y / sqrt(mean(y^2) + eps) * w with y = sum_p partials[p, t, :] (in order): a branch's output, given as
 // the partial sums of its last product, normalised and added to the stream in one pass.
+// With `bias` (or null) y also holds a bias of the product, added after the sums.
 __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, const float* __restrict__ partials, int n_partials,
-                                                       size_t partial_stride, const float* __restrict__ w, int d, float eps) {
+                                                       size_t partial_stride, const float* __restrict__ w, int d, float eps,
+                                                       const float* __restrict__ bias) {
     __shared__ float scratch[4];
     extern __shared__ float vals[];  // d floats: the summed row
     const size_t r = blockIdx.x;
@@ -212,6 +214,7 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, co
                 for (int k = 0; k < 8; ++k) v += q[k];
             }
             for (; p < n_partials; ++p) v += *reinterpret_cast<const f32x4*>(src + (size_t)p * partial_stride);
+            if (bias) v += *reinterpret_cast<const f32x4*>(bias + c);
             *reinterpret_cast<f32x4*>(vals + c) = v;
             ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         }
@@ -220,6 +223,7 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, co
             const float* src = partials + r * d + c;
             float v = 0.f;
             for (int p = 0; p < n_partials; ++p) v += src[(size_t)p * partial_stride];
+            if (bias) v += bias[c];
             vals[c] = v;
             ss += v * v;
         }
@@ -228,6 +232,93 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, co
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);
     float* dst = x + r * d;
     for (int c = threadIdx.x; c < d; c += 256) dst[c] += vals[c] * inv * w[c];
+}
+
+// Two branches side by side, each given as the partial sums of its last product: every branch's sum is normalised with
+// a weight of its own, half their sum is normalised again, and that is added to the stream:
+// y = (rms(a) * wa + rms(b) * wb) / 2;  x[t, :] += rms(y) * w.
+__global__ __launch_bounds__(256) void pair_norm_add_kernel(float* __restrict__ x, const float* __restrict__ pa, int na,
+                                                            const float* __restrict__ wa, const float* __restrict__ pb, int nb,
+                                                            const float* __restrict__ wb, size_t partial_stride,
+                                                            const float* __restrict__ w, int d, float eps) {
+    __shared__ float scratch[4];
+    extern __shared__ float vals[];  // 2 d floats: the two summed rows
+    float* va = vals;
+    float* vb = vals + d;
+    const size_t r = blockIdx.x;
+    float sa = 0.f, sb = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float a = 0.f, b = 0.f;
+        for (int p = 0; p < na; ++p) a += pa[(size_t)p * partial_stride + r * d + c];
+        for (int p = 0; p < nb; ++p) b += pb[(size_t)p * partial_stride + r * d + c];
+        va[c] = a;
+        vb[c] = b;
+        sa += a * a;
+        sb += b * b;
+    }
+    sa = block_sum<256>(sa, scratch);
+    sb = block_sum<256>(sb, scratch);
+    const float ia = 1.0f / sqrtf(sa / (float)d + eps), ib = 1.0f / sqrtf(sb / (float)d + eps);
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {  // a thread meets its own columns again: no barrier in between
+        const float y = 0.5f * (va[c] * ia * wa[c] + vb[c] * ib * wb[c]);
+        va[c] = y;
+        ss += y * y;
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    float* dst = x + r * d;
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] += va[c] * inv * w[c];
+}
+
+// out[t, c] = act(in[t, c]) * in[t, n + c]: the gated product of a feed-forward whose gate and up projections were one
+// product with biases, left as 32-bit sums
+__global__ __launch_bounds__(256) void gate_mul_kernel(const float* __restrict__ in, elem_t* __restrict__ out, int n, int act) {
+    const size_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < n; c += 256)
+        out[t * n + c] = from_f32<elem_t>(gate_activation(in[t * 2 * n + c], act) * in[t * 2 * n + n + c]);
+}
+
+// out[t, :] = the stream's row in the element type: the input of a branch that reads the stream as it is.
+__global__ __launch_bounds__(256) void round_rows_kernel(const float* __restrict__ x, elem_t* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = from_f32<elem_t>(x[i]);
+}
+
+// x[t, :] = float(table[tokens[t], :]) + float(pairs[row(t), :]) with row(t) = (previous * mul_prev + tokens[t] * mul_cur) mod
+// buckets, and row `buckets` for a request's first token.  The previous token is the row before in the step, or, for the
+// first row of a request's portion, what the request's slot of `prev [slots]` holds.
+__global__ __launch_bounds__(256) void embed_pair_kernel(const int* __restrict__ tokens, const elem_t* __restrict__ table,
+                                                         const elem_t* __restrict__ pairs, const int* __restrict__ prev,
+                                                         const int* __restrict__ seq_q_start, const int* __restrict__ seq_pos0,
+                                                         const int* __restrict__ seq_slot, int S, float* __restrict__ x, int d,
+                                                         long mul_prev, long mul_cur, long buckets) {
+    const int t = blockIdx.x;
+    int lo = 0, hi = S - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (seq_q_start[mid] <= t) lo = mid;
+        else hi = mid - 1;
+    }
+    const int j = t - seq_q_start[lo];
+    const int tok = tokens[t];
+    long row = buckets;
+    if (seq_pos0[lo] + j > 0) {
+        const int before = j > 0 ? tokens[t - 1] : prev[seq_slot[lo]];
+        row = ((long)before * mul_prev + (long)tok * mul_cur) % buckets;
+    }
+    const elem_t* a = table + (size_t)tok * d;
+    const elem_t* b = pairs + (size_t)row * d;
+    float* dst = x + (size_t)t * d;
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = to_f32(a[c]) + to_f32(b[c]);
+}
+
+// prev[slot of request s] = the last token of its rows in this step
+__global__ __launch_bounds__(256) void last_token_kernel(const int* __restrict__ tokens, const int* __restrict__ seq_q_start,
+                                                         const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot, int S,
+                                                         int* __restrict__ prev) {
+    const int s = blockIdx.x * 256 + threadIdx.x;
+    if (s < S && seq_q_len[s] > 0) prev[seq_slot[s]] = tokens[seq_q_start[s] + seq_q_len[s] - 1];
 }
 
 // v = logits * scale;  logits = cap > 0 ? cap * tanh(v / cap) : v
@@ -496,8 +587,56 @@ extern "C" int ms_norm_add(float* x, const float* partials, int n_partials, cons
     MS_REQUIRE(d <= MAX_ROW_FLOATS, "norm_add: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
     MS_REQUIRE(x && partials && w, "norm_add: a buffer is missing");
     hipLaunchKernelGGL(norm_add_kernel, dim3(T), dim3(256), (size_t)d * sizeof(float), stream, x, partials, n_partials, (size_t)T * d, w,
-                       d, eps);
+                       d, eps, (const float*)nullptr);
     return check_launch("norm_add");
+}
+
+extern "C" int ms_norm_add_bias(float* x, const float* partials, int n_partials, const float* bias, const float* w, int T, int d,
+                                float eps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && n_partials > 0, "norm_add: empty problem T=%d d=%d with %d sums", T, d, n_partials);
+    MS_REQUIRE(d <= MAX_ROW_FLOATS, "norm_add: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
+    MS_REQUIRE(x && partials && w, "norm_add: a buffer is missing");
+    hipLaunchKernelGGL(norm_add_kernel, dim3(T), dim3(256), (size_t)d * sizeof(float), stream, x, partials, n_partials, (size_t)T * d, w,
+                       d, eps, bias);
+    return check_launch("norm_add");
+}
+
+extern "C" int ms_pair_norm_add(float* x, const float* pa, int na, const float* wa, const float* pb, int nb, const float* wb,
+                                const float* w, int T, int d, float eps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && na > 0 && nb > 0, "pair_norm_add: empty problem T=%d d=%d with %d and %d sums", T, d, na, nb);
+    MS_REQUIRE(2 * d <= MAX_ROW_FLOATS, "pair_norm_add: width %d exceeds half the row buffer of %d", d, MAX_ROW_FLOATS);
+    MS_REQUIRE(x && pa && pb && wa && wb && w, "pair_norm_add: a buffer is missing");
+    hipLaunchKernelGGL(pair_norm_add_kernel, dim3(T), dim3(256), (size_t)2 * d * sizeof(float), stream, x, pa, na, wa, pb, nb, wb,
+                       (size_t)T * d, w, d, eps);
+    return check_launch("pair_norm_add");
+}
+
+extern "C" int ms_gate_mul(const float* in, void* out, int T, int n, int act, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && n > 0 && in && out, "gate_mul: empty problem T=%d n=%d", T, n);
+    MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gate_mul: activation %d", act);
+    hipLaunchKernelGGL(gate_mul_kernel, dim3(T), dim3(256), 0, stream, in, (elem_t*)out, n, act);
+    return check_launch("gate_mul");
+}
+
+extern "C" int ms_round_rows(const float* x, void* out, long n, hipStream_t stream) {
+    MS_REQUIRE(n > 0 && x && out, "round_rows: empty problem");
+    hipLaunchKernelGGL(round_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, (elem_t*)out, (size_t)n);
+    return check_launch("round_rows");
+}
+
+extern "C" int ms_embed_pair(const int* tokens, const void* table, const void* pairs, int* prev, const int* seq_q_start,
+                             const int* seq_q_len, const int* seq_pos0, const int* seq_slot, int S, float* x, int T, int d,
+                             long mul_prev, long mul_cur, long buckets, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && S > 0, "embed_pair: empty problem T=%d d=%d S=%d", T, d, S);
+    MS_REQUIRE(buckets > 0 && mul_prev >= 0 && mul_cur >= 0 && mul_prev < (1L << 31) && mul_cur < (1L << 31),
+               "embed_pair: %ld buckets, multipliers %ld and %ld", buckets, mul_prev, mul_cur);
+    hipLaunchKernelGGL(embed_pair_kernel, dim3(T), dim3(256), 0, stream, tokens, (const elem_t*)table, (const elem_t*)pairs,
+                       (const int*)prev, seq_q_start, seq_pos0, seq_slot, S, x, d, mul_prev, mul_cur, buckets);
+    int rc = check_launch("embed_pair");
+    if (rc) return rc;
+    hipLaunchKernelGGL(last_token_kernel, dim3((unsigned)ceil_div(S, 256)), dim3(256), 0, stream, tokens, seq_q_start, seq_q_len,
+                       seq_slot, S, prev);
+    return check_launch("last_token");
 }
 
 extern "C" int ms_softcap(float* logits, long n, float scale, float cap, hipStream_t stream) {

@@ -1,0 +1,385 @@
+// Linear recurrences with gates that depend on the token, and what surrounds them: a short causal convolution over
+// 32-bit sums with a state, the real-gated linear recurrent unit (gates from block-diagonal maps of the convolved
+// input, S <- a S + sqrt(1 - a^2) (i * u) with a = exp(-c r softplus(lam))), the mix of a token with the one before
+// it, and time mixing with a decay per key channel and token (S <- diag(w) S + k v^T, read with a bonus for the
+// current token), whose heads are divided by their root mean square, weighted and gated in the same kernel.
+//
+// A step's rows are the tokens of several requests, each request's rows contiguous and in order (seq_q_start,
+// seq_q_len); a request's state lives in slot seq_slot[s] of arrays [slots, ...] of 32-bit floats, is read at the start
+// of the request's rows and written back after its last.  Gates, decays and their logarithms, exponentials, the states
+// and every sum are 32-bit in every build; the element type stores what the next matrix product reads.  A row's result
+// depends on its own request alone, and on how its tokens were cut into steps not at all: every walk is token after
+// token in the same order.
+#include "common.cuh"
+
+namespace ms {
+
+__device__ __forceinline__ int seq_of_row(int t, const int* __restrict__ seq_q_start, int S) {
+    int lo = 0, hi = S - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (seq_q_start[mid] <= t) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+
+constexpr int MAX_TAPS = 16;
+
+// ---- causal convolution over 32-bit sums -------------------------------------------------
+// u[t, c] = bias_in[c] + sum_p in[p, t, col0 + c]: a projection's output, given as partial sums;
+// out[t, c] = bias_out[c] + sum_k w[c, k] * u[t - (taps - 1 - k), c].  An input before the step's first row of the
+// request comes from state [slots, taps - 1, C] (oldest first), which holds zeros before the request's start.
+struct ConvArgs {
+    const float* in;
+    int n_partials;
+    size_t partial_stride;
+    int ld, col0;
+    const float* bias_in;   // [C] or null
+    const float* w;         // [C, taps]
+    const float* bias_out;  // [C] or null
+    float* state;           // [slots, taps - 1, C]
+    const int* seq_q_start;
+    const int* seq_q_len;
+    const int* seq_slot;
+    int S;
+    float* out;             // [T, ld_out], columns out0 onwards
+    int ld_out, out0;
+    int C, taps;
+};
+
+__device__ __forceinline__ float conv_input(const ConvArgs& a, int t, int c) {
+    float v = a.bias_in ? a.bias_in[c] : 0.f;
+    const float* src = a.in + (size_t)t * a.ld + a.col0 + c;
+    for (int p = 0; p < a.n_partials; ++p) v += src[p * a.partial_stride];
+    return v;
+}
+
+__global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs a) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.C) return;
+    const int s = seq_of_row(t, a.seq_q_start, a.S);
+    const int j = t - a.seq_q_start[s];
+    const int keep = a.taps - 1;
+    const float* st = a.state + (size_t)a.seq_slot[s] * keep * a.C;
+    float acc = a.bias_out ? a.bias_out[c] : 0.f;
+    for (int k = 0; k < a.taps; ++k) {
+        const int back = keep - k, idx = j - back;
+        const float v = idx >= 0 ? conv_input(a, t - back, c) : st[(size_t)(keep + idx) * a.C + c];
+        acc += a.w[(size_t)c * a.taps + k] * v;
+    }
+    a.out[(size_t)t * a.ld_out + a.out0 + c] = acc;
+}
+
+// The state after the step: the last taps - 1 inputs of each request, old ones where the step brought fewer.
+__global__ __launch_bounds__(256) void conv_rows_state_kernel(ConvArgs a) {
+    const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.C) return;
+    const int n = a.seq_q_len[s], q0 = a.seq_q_start[s], keep = a.taps - 1;
+    float* st = a.state + (size_t)a.seq_slot[s] * keep * a.C;
+    float v[MAX_TAPS];
+    for (int i = 0; i < keep; ++i) {
+        const int idx = n - keep + i;  // among the step's rows; negative: an older input
+        v[i] = idx >= 0 ? conv_input(a, q0 + idx, c) : st[(size_t)(keep + idx) * a.C + c];
+    }
+    for (int i = 0; i < keep; ++i) st[(size_t)i * a.C + c] = v[i];
+}
+
+// ---- the gated linear recurrent unit ------------------------------------------------------
+// Gates: the channels are cut into B blocks of bw; r = sigmoid(Wa[b] u_b + ba), i = sigmoid(Wi[b] u_b + bi);
+// log a = -c r softplus(lam);  a = exp(log a);  drive = sqrt(1 - a^2) * i * u.  The weights come transposed,
+// [B, bw (in), bw (out)], so that the threads of a wave, which are outputs, read neighbouring numbers.  A block of
+// threads takes GATE_ROWS rows of one block of channels: a weight is read once for all of them.
+constexpr int GATE_ROWS = 8;
+struct GateArgs {
+    const float* u;        // [T, C]
+    const elem_t* wa_t;    // [B, bw, bw] transposed
+    const elem_t* wi_t;
+    const float* ba;       // [C]
+    const float* bi;       // [C]
+    const float* lam;      // [C]
+    float c;               // the factor in the decay's exponent
+    float* a_out;          // [T, C]
+    float* drive_out;      // [T, C]
+    int T, C, bw;
+};
+
+__global__ __launch_bounds__(256) void lru_gates_kernel(GateArgs g) {
+    extern __shared__ float us[];  // [GATE_ROWS][bw]
+    const int t0 = blockIdx.x * GATE_ROWS, b = blockIdx.y, bw = g.bw;
+    const int nr = min(GATE_ROWS, g.T - t0);
+    for (int i = threadIdx.x; i < GATE_ROWS * bw; i += 256) {
+        const int r = i / bw, k = i - r * bw;
+        us[i] = r < nr ? g.u[(size_t)(t0 + r) * g.C + b * bw + k] : 0.f;
+    }
+    __syncthreads();
+    const elem_t* wa = g.wa_t + (size_t)b * bw * bw;
+    const elem_t* wi = g.wi_t + (size_t)b * bw * bw;
+    for (int o = threadIdx.x; o < bw; o += 256) {
+        float ar[GATE_ROWS], ai[GATE_ROWS];
+#pragma unroll
+        for (int r = 0; r < GATE_ROWS; ++r) ar[r] = ai[r] = 0.f;
+        for (int k = 0; k < bw; ++k) {
+            const float fa = to_f32(wa[(size_t)k * bw + o]), fi = to_f32(wi[(size_t)k * bw + o]);
+#pragma unroll
+            for (int r = 0; r < GATE_ROWS; ++r) {
+                const float uv = us[r * bw + k];
+                ar[r] += fa * uv;
+                ai[r] += fi * uv;
+            }
+        }
+        const int c = b * bw + o;
+        const float sp = softplus_f(g.lam[c]), ba = g.ba[c], bi = g.bi[c];
+#pragma unroll
+        for (int r = 0; r < GATE_ROWS; ++r) {
+            if (r < nr) {
+                const float rg = sigmoid_f(ar[r] + ba), ig = sigmoid_f(ai[r] + bi);
+                const float log_a = -g.c * rg * sp;
+                const float av = expf(log_a);
+                // 1 - a^2 = -expm1(2 log a): no cancellation where a is close to one
+                const float drive = sqrtf(-expm1f(2.0f * log_a)) * ig * us[r * bw + o];
+                g.a_out[(size_t)(t0 + r) * g.C + c] = av;
+                g.drive_out[(size_t)(t0 + r) * g.C + c] = drive;
+            }
+        }
+    }
+}
+
+// The recurrence, a channel a thread, a request's rows in order: S <- a S + drive;  out = S * gelu_tanh(y + by), with y
+// the other branch's projection in the element type (columns ycol onwards of rows of ld elements).
+constexpr int LRU_AHEAD = 8;
+__global__ __launch_bounds__(64) void lru_scan_kernel(const float* __restrict__ a, const float* __restrict__ drive,
+                                                      const elem_t* __restrict__ y, int ldy, int ycol, const float* __restrict__ by,
+                                                      float* __restrict__ state, const int* __restrict__ seq_q_start,
+                                                      const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot,
+                                                      elem_t* __restrict__ out, int C) {
+    const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+    if (c >= C) return;
+    const int q0 = seq_q_start[s], n = seq_q_len[s];
+    if (n <= 0) return;
+    float* st = state + (size_t)seq_slot[s] * C + c;
+    float S = *st;
+    const float bias = by ? by[c] : 0.f;
+    for (int j0 = 0; j0 < n; j0 += LRU_AHEAD) {
+        float av[LRU_AHEAD], dv[LRU_AHEAD], yv[LRU_AHEAD];
+#pragma unroll
+        for (int k = 0; k < LRU_AHEAD; ++k) {  // a batch of loads, then the chain
+            const int t = q0 + min(j0 + k, n - 1);
+            av[k] = a[(size_t)t * C + c];
+            dv[k] = drive[(size_t)t * C + c];
+            yv[k] = to_f32(y[(size_t)t * ldy + ycol + c]);
+        }
+#pragma unroll
+        for (int k = 0; k < LRU_AHEAD; ++k) {
+            if (j0 + k < n) {
+                S = av[k] * S + dv[k];
+                out[(size_t)(q0 + j0 + k) * C + c] = from_f32<elem_t>(S * gelu_tanh_f(yv[k] + bias));
+            }
+        }
+    }
+    *st = S;
+}
+
+// ---- the mix of a token with the one before it ---------------------------------------------
+// out[m, t, :] = x[t] + (x[t - 1] - x[t]) * mu[m, :] for M mixes, in the element type; the row before a request's first
+// row of the step comes from prev [slots, d] (zeros at the request's start).
+__global__ __launch_bounds__(256) void shift_mix_kernel(const float* __restrict__ x, const float* __restrict__ prev,
+                                                        const float* __restrict__ mu, int M, const int* __restrict__ seq_q_start,
+                                                        const int* __restrict__ seq_slot, int S, elem_t* __restrict__ out, int T, int d) {
+    const int t = blockIdx.x;
+    const int s = seq_of_row(t, seq_q_start, S);
+    const float* before = t > seq_q_start[s] ? x + (size_t)(t - 1) * d : prev + (size_t)seq_slot[s] * d;
+    const float* cur = x + (size_t)t * d;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        const float v = cur[c], dlt = before[c] - v;
+        for (int m = 0; m < M; ++m) out[((size_t)m * T + t) * d + c] = from_f32<elem_t>(v + dlt * mu[(size_t)m * d + c]);
+    }
+}
+
+// prev[slot of request s] = its last row of the step
+__global__ __launch_bounds__(256) void last_row_kernel(const float* __restrict__ x, float* __restrict__ prev,
+                                                       const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+                                                       const int* __restrict__ seq_slot, int d) {
+    const int s = blockIdx.x, n = seq_q_len[s];
+    if (n <= 0) return;
+    const float* src = x + (size_t)(seq_q_start[s] + n - 1) * d;
+    float* dst = prev + (size_t)seq_slot[s] * d;
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = src[c];
+}
+
+// out = act(in) in the element type: the bottleneck of a low-rank map between its two products (0: tanh)
+__global__ __launch_bounds__(256) void tanh_rows_kernel(const float* __restrict__ in, elem_t* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = from_f32<elem_t>(tanhf(in[i]));
+}
+
+// ---- time mixing with a decay per key channel and token ----------------------------------------
+// Per head, state S [d (key channel), d (value channel)]; token by token
+//   o[j] = sum_i r[i] (S[i, j] + u[i] k[i] v[j]);   S[i, j] <- w[i] S[i, j] + k[i] v[j],   w = exp(-exp(z + w0)).
+// A thread is a value channel j and holds its column of S in registers (DP of them, the head size rounded up to a
+// multiple of 16; the rows beyond d stay zero).  Then, in the same kernel: o / sqrt(mean_j o^2 + eps) * norm[h, j] *
+// silu(gate[t, h, j]), rounded to the element type for the output projection.
+struct WkvArgs {
+    const elem_t* r;     // [T, H * d]
+    const elem_t* k;
+    const elem_t* v;
+    const elem_t* gate;  // [T, H * d] before its SiLU
+    const float* z;      // [T, H * d]: the decay's inner logarithm before its offset
+    const float* w0;     // [H * d]
+    const float* u;      // [H * d]
+    const float* norm;   // [H * d]
+    float eps;
+    float* state;        // [slots, H, d, d]
+    const int* seq_q_start;
+    const int* seq_q_len;
+    const int* seq_slot;
+    elem_t* out;         // [T, H * d]
+    int H, d;
+};
+
+template <int DP>
+__global__ __launch_bounds__(DP <= 64 ? 64 : 128) void wkv_kernel(WkvArgs a) {
+    constexpr int NT = DP <= 64 ? 64 : 128;
+    __shared__ float rs[2][DP], ks[2][DP], ws[2][DP];
+    __shared__ float scratch[NT / 64];
+    const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x, d = a.d, row = a.H * d;
+    const int q0 = a.seq_q_start[s], n = a.seq_q_len[s];
+    if (n <= 0) return;
+    const bool live = j < d;
+    float* st = a.state + (((size_t)a.seq_slot[s] * a.H + h) * d) * d;
+    float S[DP];
+#pragma unroll
+    for (int i = 0; i < DP; ++i) S[i] = (live && i < d) ? st[(size_t)i * d + j] : 0.f;
+    const int col = h * d + (live ? j : 0);
+    const float w0 = a.w0[col], uj = a.u[col], nw = a.norm[col];
+    auto stage = [&](int b, int t) {  // this thread's key channel of token t
+        if (j < DP) {
+            const size_t at = (size_t)t * row + col;
+            rs[b][j] = live ? to_f32(a.r[at]) : 0.f;
+            ks[b][j] = live ? to_f32(a.k[at]) : 0.f;
+            ws[b][j] = live ? expf(-expf(a.z[at] + w0)) : 0.f;
+        }
+    };
+    // the bonus belongs to the key channel: u[i] k[i]; kept beside k in LDS as r[i] u[i] k[i] would need r first
+    __shared__ float us[DP];
+    if (j < DP) us[j] = live ? uj : 0.f;
+    stage(0, q0);
+    __syncthreads();
+    for (int jt = 0; jt < n; ++jt) {
+        const int b = jt & 1, t = q0 + jt;
+        if (jt + 1 < n) stage(b ^ 1, t + 1);
+        const float vj = live ? to_f32(a.v[(size_t)t * row + col]) : 0.f;
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DP; ++i) {
+            const float kv = ks[b][i] * vj;
+            o += rs[b][i] * (S[i] + us[i] * kv);
+            S[i] = ws[b][i] * S[i] + kv;
+        }
+        float ss = live ? o * o : 0.f;
+        if constexpr (NT == 64) {
+            ss = wave_sum(ss);
+            __syncthreads();  // the next token's stage is written; this token's has been read by everyone
+        } else {
+            ss = block_sum<NT>(ss, scratch);  // its barriers do the same
+        }
+        if (live) {
+            const float g = to_f32(a.gate[(size_t)t * row + col]);
+            const float y = o / sqrtf(ss / (float)d + a.eps) * nw * (g / (1.0f + expf(-g)));
+            a.out[(size_t)t * row + col] = from_f32<elem_t>(y);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DP; ++i)
+            if (i < d) st[(size_t)i * d + j] = S[i];
+    }
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+extern "C" int ms_linrec_max_taps() { return MAX_TAPS; }
+extern "C" int ms_wkv_max_dim() { return 128; }
+
+// One launch for the convolution and one for the state, in this order: the first reads the state that the second
+// replaces.  `out` may not alias `in`.
+extern "C" int ms_conv_sums(const float* in, int n_partials, long partial_stride, int ld, int col0, const float* bias_in, const float* w,
+                            const float* bias_out, float* state, const int* seq_q_start, const int* seq_q_len, const int* seq_slot,
+                            int S, float* out, int ld_out, int out0, int T, int C, int taps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && C > 0 && S > 0 && n_partials > 0, "conv_sums: empty problem T=%d C=%d S=%d", T, C, S);
+    MS_REQUIRE(taps >= 1 && taps <= MAX_TAPS, "conv_sums: %d taps (1 to %d)", taps, MAX_TAPS);
+    MS_REQUIRE(col0 >= 0 && col0 + C <= ld && out0 >= 0 && out0 + C <= ld_out, "conv_sums: columns %d..%d of %d, %d..%d of %d", col0,
+               col0 + C, ld, out0, out0 + C, ld_out);
+    MS_REQUIRE(taps == 1 || state, "conv_sums: %d taps need a state", taps);
+    ConvArgs a{in, n_partials, (size_t)partial_stride, ld, col0, bias_in, w, bias_out, state, seq_q_start, seq_q_len, seq_slot, S,
+               out, ld_out, out0, C, taps};
+    hipLaunchKernelGGL(conv_rows_kernel, dim3(T, ceil_div(C, 256)), dim3(256), 0, stream, a);
+    int rc = check_launch("conv_sums");
+    if (rc || taps == 1) return rc;
+    hipLaunchKernelGGL(conv_rows_state_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, a);
+    return check_launch("conv_sums_state");
+}
+
+extern "C" int ms_lru_gates(const float* u, const void* wa_t, const void* wi_t, const float* ba, const float* bi, const float* lam,
+                            float c, float* a_out, float* drive_out, int T, int C, int blocks, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && C > 0 && blocks > 0 && C % blocks == 0, "lru_gates: %d channels in %d blocks, %d rows", C, blocks, T);
+    const int bw = C / blocks;
+    const size_t lds = (size_t)GATE_ROWS * bw * sizeof(float);
+    MS_REQUIRE(lds <= 64 * 1024, "lru_gates: blocks of %d channels exceed the rows' place in LDS", bw);
+    GateArgs g{u, (const elem_t*)wa_t, (const elem_t*)wi_t, ba, bi, lam, c, a_out, drive_out, T, C, bw};
+    hipLaunchKernelGGL(lru_gates_kernel, dim3(ceil_div(T, GATE_ROWS), blocks), dim3(256), lds, stream, g);
+    return check_launch("lru_gates");
+}
+
+extern "C" int ms_lru_scan(const float* a, const float* drive, const void* y, int ldy, int ycol, const float* by, float* state,
+                           const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, void* out, int C,
+                           hipStream_t stream) {
+    MS_REQUIRE(S > 0 && C > 0 && ycol >= 0 && ycol + C <= ldy, "lru_scan: %d requests, %d channels at column %d of %d", S, C, ycol, ldy);
+    hipLaunchKernelGGL(lru_scan_kernel, dim3(S, ceil_div(C, 64)), dim3(64), 0, stream, a, drive, (const elem_t*)y, ldy, ycol, by,
+                       state, seq_q_start, seq_q_len, seq_slot, (elem_t*)out, C);
+    return check_launch("lru_scan");
+}
+
+extern "C" int ms_shift_mix(const float* x, float* prev, const float* mu, int M, const int* seq_q_start, const int* seq_q_len,
+                            const int* seq_slot, int S, void* out, int T, int d, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && S > 0 && M > 0, "shift_mix: empty problem T=%d d=%d S=%d M=%d", T, d, S, M);
+    hipLaunchKernelGGL(shift_mix_kernel, dim3(T), dim3(256), 0, stream, x, (const float*)prev, mu, M, seq_q_start, seq_slot, S,
+                       (elem_t*)out, T, d);
+    int rc = check_launch("shift_mix");
+    if (rc) return rc;
+    hipLaunchKernelGGL(last_row_kernel, dim3(S), dim3(256), 0, stream, x, prev, seq_q_start, seq_q_len, seq_slot, d);
+    return check_launch("last_row");
+}
+
+extern "C" int ms_tanh_rows(const float* in, void* out, long n, hipStream_t stream) {
+    MS_REQUIRE(n > 0, "tanh_rows: empty problem");
+    hipLaunchKernelGGL(tanh_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, in, (elem_t*)out, (size_t)n);
+    return check_launch("tanh_rows");
+}
+
+extern "C" int ms_wkv(const void* r, const void* k, const void* v, const void* gate, const float* z, const float* w0, const float* u,
+                      const float* norm, float eps, float* state, const int* seq_q_start, const int* seq_q_len, const int* seq_slot,
+                      int S, void* out, int H, int d, hipStream_t stream) {
+    MS_REQUIRE(S > 0 && H > 0 && d > 0 && d <= 128, "wkv: %d requests, %d heads of %d (at most 128)", S, H, d);
+    WkvArgs a{(const elem_t*)r, (const elem_t*)k, (const elem_t*)v, (const elem_t*)gate, z, w0, u, norm, eps, state,
+              seq_q_start, seq_q_len, seq_slot, (elem_t*)out, H, d};
+    const dim3 grid(S, H);
+    const int dp = ceil_div(d, 16) * 16;
+    switch (dp) {
+        case 16: hipLaunchKernelGGL(wkv_kernel<16>, grid, dim3(64), 0, stream, a); break;
+        case 32: hipLaunchKernelGGL(wkv_kernel<32>, grid, dim3(64), 0, stream, a); break;
+        case 48: hipLaunchKernelGGL(wkv_kernel<48>, grid, dim3(64), 0, stream, a); break;
+        case 64: hipLaunchKernelGGL(wkv_kernel<64>, grid, dim3(64), 0, stream, a); break;
+        case 80: hipLaunchKernelGGL(wkv_kernel<80>, grid, dim3(128), 0, stream, a); break;
+        case 96: hipLaunchKernelGGL(wkv_kernel<96>, grid, dim3(128), 0, stream, a); break;
+        case 112: hipLaunchKernelGGL(wkv_kernel<112>, grid, dim3(128), 0, stream, a); break;
+        default: hipLaunchKernelGGL(wkv_kernel<128>, grid, dim3(128), 0, stream, a); break;
+    }
+    return check_launch("wkv");
+}

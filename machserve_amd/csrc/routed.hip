@@ -1,0 +1,105 @@
+// A feed-forward of many small experts of which a token uses a few: the router, and the experts' activation.
+//
+// The router's logits are 32-bit sums of 32-bit weights times the rows as the feed-forward's products read them (in the
+// element type, which the 32-bit build does not round); a row's `top` largest logits choose its experts (the lower
+// index wins a tie), and their weights are the softmax over the chosen logits alone.  The experts' up projections are one
+// matrix [experts * ff (+ shared), width] and their down projections one matrix [width, experts * ff (+ shared)], so the
+// weighted sum of the chosen experts' outputs is ONE product over activations in which an expert's columns are
+// act(up) * (the row's weight for that expert), zero for an expert the row did not choose, and the columns of an
+// expert that every row uses (beyond experts * ff) carry weight one.  Nothing here depends on what else is in the step.
+#include "common.cuh"
+
+namespace ms {
+
+constexpr int MAX_EXPERTS = 1024;
+
+// gates[t, e] = the row's weight for expert e, 0 where it was not chosen.  One block a row: a wave a logit in turn.
+__global__ __launch_bounds__(256) void route_kernel(const elem_t* __restrict__ x, const float* __restrict__ w,
+                                                    const float* __restrict__ bias, float* __restrict__ gates, int d, int E, int top) {
+    __shared__ float z[MAX_EXPERTS];
+    __shared__ float chosen_z[64];
+    __shared__ int chosen_e[64];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const elem_t* row = x + (size_t)t * d;
+    for (int e = wave; e < E; e += 4) {
+        const float* we = w + (size_t)e * d;
+        float acc = 0.f;
+        for (int c = lane; c < d; c += 64) acc += to_f32(row[c]) * we[c];
+        acc = wave_sum(acc);
+        if (lane == 0) z[e] = acc + (bias ? bias[e] : 0.f);
+    }
+    __syncthreads();
+    if (wave == 0) {
+        // `top` rounds of a maximum over the wave; the winner leaves the list
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY;
+            int at = MAX_EXPERTS;
+            for (int e = lane; e < E; e += 64)
+                if (z[e] > best) { best = z[e]; at = e; }
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, WAVE);
+                const int oa = __shfl_xor(at, o, WAVE);
+                if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+            }
+            if (lane == 0) {
+                chosen_z[k] = best;
+                chosen_e[k] = at;
+                if (at < E) z[at] = -INFINITY;
+            }
+            __builtin_amdgcn_wave_barrier();
+            __threadfence_block();
+        }
+    }
+    __syncthreads();
+    float* g = gates + (size_t)t * E;
+    for (int e = threadIdx.x; e < E; e += 256) g[e] = 0.f;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float m = chosen_z[0];  // the first chosen is the largest
+        float sum = 0.f;
+        for (int k = 0; k < top; ++k) sum += expf(chosen_z[k] - m);
+        for (int k = 0; k < top; ++k)
+            if (chosen_e[k] < E) g[chosen_e[k]] = expf(chosen_z[k] - m) / sum;
+    }
+}
+
+// act: 0 the exact GELU (erf), 1 its tanh form, 2 SiLU
+__device__ __forceinline__ float expert_activation(float z, int act) {
+    if (act == 0) return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+    if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z / (1.0f + expf(-z));
+}
+
+// a[t, c] = act(up[t, c]) * gates[t, c / ff] for c < E * ff, act(up[t, c]) beyond (experts that every row uses)
+__global__ __launch_bounds__(256) void expert_act_kernel(const float* __restrict__ up, const float* __restrict__ gates,
+                                                         elem_t* __restrict__ out, int n, int E, int ff, int act) {
+    const int t = blockIdx.x;
+    const float* g = gates + (size_t)t * E;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const int e = c / ff;
+        const float w = e < E ? g[e] : 1.0f;
+        // an expert the row did not choose contributes an exact zero, whatever its product holds
+        out[(size_t)t * n + c] = from_f32<elem_t>(w != 0.f ? expert_activation(up[(size_t)t * n + c], act) * w : 0.f);
+    }
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+extern "C" int ms_route_max_experts() { return MAX_EXPERTS; }
+
+extern "C" int ms_route(const void* x, const float* w, const float* bias, float* gates, int T, int d, int E, int top,
+                        hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && E > 0 && E <= MAX_EXPERTS, "route: %d rows of %d over %d experts (at most %d)", T, d, E, MAX_EXPERTS);
+    MS_REQUIRE(top >= 1 && top <= E && top <= 64, "route: %d of %d experts a row (at most 64)", top, E);
+    hipLaunchKernelGGL(route_kernel, dim3(T), dim3(256), 0, stream, (const elem_t*)x, w, bias, gates, d, E, top);
+    return check_launch("route");
+}
+
+extern "C" int ms_expert_act(const float* up, const float* gates, void* out, int T, int n, int E, int ff, int act, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && n > 0 && E >= 0 && ff > 0 && (long)E * ff <= n, "expert_act: %d columns for %d experts of %d", n, E, ff);
+    MS_REQUIRE(act >= 0 && act <= 2, "expert_act: activation %d", act);
+    hipLaunchKernelGGL(expert_act_kernel, dim3(T), dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
+    return check_launch("expert_act");
+}

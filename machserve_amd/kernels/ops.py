@@ -435,9 +435,9 @@ class HipOps:
         nd = build.attention_tile_for(hd)
         if nd not in self._attn:
             lib = self._load(build.ensure_library("attention", self.elem, nd))
-            self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_ex_nd{nd}"),
+            self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_mask_nd{nd}"),
                               getattr(lib, f"ms_attention_rows_per_block_nd{nd}")(),
-                              getattr(lib, f"ms_decode_attention_ex_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")(),
+                              getattr(lib, f"ms_decode_attention_mask_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")(),
                               getattr(lib, f"ms_decode_attention_fused_nd{nd}"))
         return self._attn[nd]
 
@@ -448,8 +448,10 @@ class HipOps:
                         seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
                         scale: float, max_key_groups: int = 0, key_splits: int = 0, sinks: Optional[torch.Tensor] = None,
-                        out_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """``sinks`` float32 ``[H]``: the softmax's denominator also holds ``exp(sinks[h])``, a term without key or value;
+                        out_gate: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
+        """``chunk`` > 0: a row at position p sees only keys from ``floor(p / chunk) * chunk`` on (chunks counted from the
+        request's position 0); ``softcap`` > 0: a scaled score s becomes ``softcap * tanh(s / softcap)`` before the softmax.
+        ``sinks`` float32 ``[H]``: the softmax's denominator also holds ``exp(sinks[h])``, a term without key or value;
         ``out_gate`` float32 ``[T, H]``: what the output of each (row, head) is multiplied by, in the kernel's last pass.
         ``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's
         choice); ``key_splits`` for that many blocks sharing them (0: the library's choice by the number of blocks
@@ -472,7 +474,7 @@ class HipOps:
             raise KernelError(f"attention: work list of shape {tuple(work.shape)}")
         out = torch.empty((T, H * hd), dtype=self.dtype, device=q.device)
         nsplit = key_splits or self._plan(f"ms_attention_splits_nd{build.attention_tile_for(hd)}", work.shape[0], KV, T, hd, page_size,
-                                          block_table.shape[1], window or 0, lib=lib)
+                                          block_table.shape[1], self._reach(window, chunk), lib=lib)
         part_o = part_ml = None
         if nsplit > 1:
             part_o = torch.empty((T, H, nsplit, hd), dtype=torch.float32, device=q.device)
@@ -481,8 +483,14 @@ class HipOps:
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
                             _c_float(scale), _c_int(max_key_groups), _c_int(T), _c_int(nsplit), _ptr(part_o), _ptr(part_ml),
-                            _ptr(sinks), _ptr(out_gate), self._stream()))
+                            _ptr(sinks), _ptr(out_gate), _c_int(chunk), _c_float(softcap), self._stream()))
         return out
+
+    @staticmethod
+    def _reach(window: Optional[int], chunk: int) -> int:
+        """How far back a row can see under a window and a chunked mask (0: all the way)."""
+        reaches = [r for r in (window or 0, chunk or 0) if r > 0]
+        return min(reaches) if reaches else 0
 
     def _want_softmax_extras(self, sinks, out_gate, T: int, H: int) -> None:
         if sinks is not None:
@@ -544,8 +552,9 @@ class HipOps:
 
     def decode_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                          seq_pos0: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
-                         scale: float, sinks: Optional[torch.Tensor] = None, out_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Attention of a step in which request ``s`` has the single row ``s`` (``sinks``, ``out_gate``: see
+                         scale: float, sinks: Optional[torch.Tensor] = None, out_gate: Optional[torch.Tensor] = None,
+                         chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
+        """Attention of a step in which request ``s`` has the single row ``s`` (``sinks``, ``out_gate``, ``chunk``, ``softcap``: see
         :meth:`paged_attention`).  The keys are cut
         into splits so that the grid fills the chip; how many follows from the number of
         requests and the width of the block table only."""
@@ -562,7 +571,7 @@ class HipOps:
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         if H // KV > self.DECODE_MAX_GROUP:
             raise KernelError(f"decode attention: {H // KV} heads per key/value head, at most {self.DECODE_MAX_GROUP}")
-        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, window, key_tile, hd)
+        nsplit = self._decode_splits(S, KV, block_table.shape[1], page_size, self._reach(window, chunk) or None, key_tile, hd)
         out = torch.empty((S, H * hd), dtype=self.dtype, device=q.device)
         part_o = part_ml = None
         if nsplit > 1:
@@ -571,7 +580,7 @@ class HipOps:
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
                             _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
                             _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _ptr(sinks), _ptr(out_gate),
-                            self._stream()))
+                            _c_int(chunk), _c_float(softcap), self._stream()))
         return out
 
     # ------------------------------------------------------------------ a branch's output, normalised, into the stream
@@ -953,6 +962,256 @@ class HipOps:
                                           _ptr(kpool), _ptr(vpool), _ptr(gate), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dp),
                                           _c_int(page_size), self._stream()))
         return q, gate
+
+    # ------------------------------------------------------------------ branches that end in a norm of their own
+    def norm_add_bias(self, x: torch.Tensor, partials: torch.Tensor, bias: Optional[torch.Tensor], weight: torch.Tensor, eps: float) -> None:
+        """``x += rmsnorm(sum(partials) + bias) * weight``: :meth:`norm_add` for a product that has a bias."""
+        if bias is None:
+            return self.norm_add(x, partials, weight, eps)
+        T, d = x.shape
+        self._want(x, torch.float32, "norm_add stream")
+        self._want(partials, torch.float32, "norm_add sums", partials.shape[0], T, d)
+        self._want(bias, torch.float32, "norm_add bias", d)
+        self._want(weight, torch.float32, "norm_add weight", d)
+        self._check(self._core, self._core.ms_norm_add_bias(_ptr(x), _ptr(partials), _c_int(partials.shape[0]), _ptr(bias), _ptr(weight),
+                                                            _c_int(T), _c_int(d), _c_float(eps), self._stream()))
+
+    def pair_norm_add(self, x: torch.Tensor, pa: torch.Tensor, wa: torch.Tensor, pb: torch.Tensor, wb: torch.Tensor, weight: torch.Tensor,
+                      eps: float) -> None:
+        """``y = (rmsnorm(sum(pa)) * wa + rmsnorm(sum(pb)) * wb) / 2;  x += rmsnorm(y) * weight``: two branches side by side,
+        each given as the float32 partial sums ``[P, T, d]`` of its last product."""
+        T, d = x.shape
+        self._want(x, torch.float32, "pair_norm_add stream")
+        self._want(pa, torch.float32, "pair_norm_add sums", pa.shape[0], T, d)
+        self._want(pb, torch.float32, "pair_norm_add sums", pb.shape[0], T, d)
+        for w in (wa, wb, weight):
+            self._want(w, torch.float32, "pair_norm_add weight", d)
+        self._check(self._core, self._core.ms_pair_norm_add(_ptr(x), _ptr(pa), _c_int(pa.shape[0]), _ptr(wa), _ptr(pb), _c_int(pb.shape[0]),
+                                                            _ptr(wb), _ptr(weight), _c_int(T), _c_int(d), _c_float(eps), self._stream()))
+
+    def gate_mul(self, sums: torch.Tensor, activation: str) -> torch.Tensor:
+        """``act(sums[:, :n]) * sums[:, n:]`` in the element type for float32 ``sums [T, 2 n]``: the gated product of a
+        feed-forward whose gate and up projections carry biases."""
+        T, n2 = sums.shape
+        self._want(sums, torch.float32, "gate_mul sums")
+        if n2 % 2:
+            raise KernelError(f"gate_mul: {n2} columns are not a gate and an up half")
+        out = torch.empty((T, n2 // 2), dtype=self.dtype, device=sums.device)
+        self._check(self._core, self._core.ms_gate_mul(_ptr(sums), _ptr(out), _c_int(T), _c_int(n2 // 2), _c_int(gate_activation_code(activation)),
+                                                       self._stream()))
+        return out
+
+    def round_rows(self, x: torch.Tensor) -> torch.Tensor:
+        """The 32-bit stream in the element type (a copy in the 32-bit build): the input of a branch that reads the stream as it is."""
+        self._want(x, torch.float32, "round_rows stream")
+        out = torch.empty(x.shape, dtype=self.dtype, device=x.device)
+        self._check(self._core, self._core.ms_round_rows(_ptr(x), _ptr(out), ctypes.c_long(x.numel()), self._stream()))
+        return out
+
+    def embed_pair(self, tokens: torch.Tensor, table: torch.Tensor, pairs: torch.Tensor, prev: torch.Tensor, seq_q_start: torch.Tensor,
+                   seq_q_len: torch.Tensor, seq_pos0: torch.Tensor, seq_slot: torch.Tensor, mul_prev: int, mul_cur: int, buckets: int) -> torch.Tensor:
+        """``table[token] + pairs[(previous * mul_prev + token * mul_cur) mod buckets]`` (row ``buckets`` for a request's
+        first token) as float32 rows; the token before a portion's first row is what ``prev [slots]`` holds, and the
+        portion's last token is left there."""
+        T, (V, d) = tokens.numel(), table.shape
+        self._want(tokens, torch.int32, "embed tokens", T)
+        self._want(table, self.dtype, "embed table")
+        self._want(pairs, self.dtype, "embed pair table", buckets + 1, d)
+        self._want(prev, torch.int32, "embed previous tokens")
+        S = self._seq_operands("embed", seq_q_start, seq_q_len, seq_slot)
+        self._want(seq_pos0, torch.int32, "embed seq_pos0", S)
+        x = torch.empty((T, d), dtype=torch.float32, device=table.device)
+        L = ctypes.c_long
+        self._check(self._core, self._core.ms_embed_pair(_ptr(tokens), _ptr(table), _ptr(pairs), _ptr(prev), _ptr(seq_q_start), _ptr(seq_q_len),
+                                                         _ptr(seq_pos0), _ptr(seq_slot), _c_int(S), _ptr(x), _c_int(T), _c_int(d), L(mul_prev),
+                                                         L(mul_cur), L(buckets), self._stream()))
+        return x
+
+    # ------------------------------------------------------------------ q, k and v finished from 32-bit rows
+    def finish_rows(self, rows: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
+                    positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot: int, neighbours: bool, slot_map: torch.Tensor,
+                    kpool: torch.Tensor, vpool: torch.Tensor, H: int, KV: int, d: int, dv: int, page_size: int) -> torch.Tensor:
+        """``rows`` float32 ``[T, >= H d + KV d + KV dv]`` hold q, k and v: an RMS norm over all of q and one over all of k
+        (weights; None: none), the rotation of the first ``rot`` numbers of every head of q and k by ``position * inv_freq``
+        (pairs of neighbours, or ``(i, i + rot / 2)``), k and v written into their pages.  Returns q ``[T, H * dp]`` in the
+        element type, ``dp`` the pools' head size (zeros beyond ``d``)."""
+        lib = self._extra_lib("convattn")
+        T, stride = rows.shape
+        self._want(rows, torch.float32, "finish rows")
+        if q_norm is not None:
+            self._want(q_norm, torch.float32, "query norm weight", H * d)
+        if k_norm is not None:
+            self._want(k_norm, torch.float32, "key norm weight", KV * d)
+        self._want(positions, torch.int32, "finish rows positions", T)
+        if inv_freq is not None:
+            self._want(inv_freq, torch.float32, "rotation frequencies", rot // 2)
+        else:
+            rot = 0
+        self._want(slot_map, torch.int32, "finish rows slot_map", T)
+        pages, _, _, dp = kpool.shape
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, dp)
+        self._want(vpool, self.dtype, "value pool", pages, KV, dp, page_size)
+        q = torch.empty((T, H * dp), dtype=self.dtype, device=rows.device)
+        self._check(lib, lib.ms_finish_rows(_ptr(rows), _c_int(stride), _ptr(q_norm), _ptr(k_norm), _c_float(eps), _ptr(positions),
+                                            _ptr(inv_freq), _c_int(rot), _c_int(int(neighbours)), _ptr(slot_map), _ptr(q), _ptr(kpool),
+                                            _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(dp),
+                                            _c_int(page_size), self._stream()))
+        return q
+
+    # ------------------------------------------------------------------ linear recurrences with gates that depend on the token
+    def linrec_limits(self) -> dict:
+        lib = self._extra_lib("linrec")
+        return {"taps": lib.ms_linrec_max_taps(), "wkv_dim": lib.ms_wkv_max_dim()}
+
+    def conv_sums(self, sums: torch.Tensor, col0: int, channels: int, bias_in: Optional[torch.Tensor], weight: torch.Tensor,
+                  bias_out: Optional[torch.Tensor], state: Optional[torch.Tensor], seq_q_start: torch.Tensor, seq_q_len: torch.Tensor,
+                  seq_slot: torch.Tensor) -> torch.Tensor:
+        """A causal convolution per channel over a projection given as float32 partial sums ``[P, T, N]`` (columns ``col0``
+        onwards, plus ``bias_in``): ``out[t] = bias_out + sum_k weight[:, k] u[t - (taps - 1 - k)]``, the inputs before a
+        request's rows of this step from ``state [slots, taps - 1, channels]``, which is brought up to date.  Float32 ``[T, channels]``."""
+        lib = self._extra_lib("linrec")
+        if sums.dim() == 2:
+            sums = sums.unsqueeze(0)
+        P, T, N = sums.shape
+        self._want(sums, torch.float32, "conv_sums input")
+        taps = weight.shape[1]
+        self._want(weight, torch.float32, "conv_sums weight", channels, taps)
+        for b in (bias_in, bias_out):
+            if b is not None:
+                self._want(b, torch.float32, "conv_sums bias", channels)
+        if taps > 1:
+            self._want(state, torch.float32, "conv_sums state", state.shape[0], taps - 1, channels)
+        else:
+            state = None
+        S = self._seq_operands("conv_sums", seq_q_start, seq_q_len, seq_slot)
+        out = torch.empty((T, channels), dtype=torch.float32, device=sums.device)
+        self._check(lib, lib.ms_conv_sums(_ptr(sums), _c_int(P), ctypes.c_long(T * N), _c_int(N), _c_int(col0), _ptr(bias_in), _ptr(weight),
+                                          _ptr(bias_out), _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out),
+                                          _c_int(channels), _c_int(0), _c_int(T), _c_int(channels), _c_int(taps), self._stream()))
+        return out
+
+    def lru_gates(self, u: torch.Tensor, wa_t: torch.Tensor, wi_t: torch.Tensor, ba: torch.Tensor, bi: torch.Tensor, lam: torch.Tensor,
+                  factor: float):
+        """Gates of the real-gated linear recurrent unit from ``u`` float32 ``[T, C]``: per block of channels
+        ``r = sigmoid(Wa u + ba)``, ``i = sigmoid(Wi u + bi)`` (weights transposed, ``[blocks, in, out]``), ``a = exp(-factor r
+        softplus(lam))``; returns float32 ``(a, sqrt(1 - a^2) i u)``."""
+        lib = self._extra_lib("linrec")
+        T, C = u.shape
+        blocks, bw, _ = wa_t.shape
+        self._want(u, torch.float32, "lru input")
+        self._want(wa_t, self.dtype, "lru gate weight", blocks, bw, bw)
+        self._want(wi_t, self.dtype, "lru gate weight", blocks, bw, bw)
+        if blocks * bw != C:
+            raise KernelError(f"lru_gates: {blocks} blocks of {bw} for {C} channels")
+        for v in (ba, bi, lam):
+            self._want(v, torch.float32, "lru gate vector", C)
+        a = torch.empty((T, C), dtype=torch.float32, device=u.device)
+        drive = torch.empty((T, C), dtype=torch.float32, device=u.device)
+        self._check(lib, lib.ms_lru_gates(_ptr(u), _ptr(wa_t), _ptr(wi_t), _ptr(ba), _ptr(bi), _ptr(lam), _c_float(factor), _ptr(a), _ptr(drive),
+                                          _c_int(T), _c_int(C), _c_int(blocks), self._stream()))
+        return a, drive
+
+    def lru_scan(self, a: torch.Tensor, drive: torch.Tensor, y: torch.Tensor, ycol: int, y_bias: Optional[torch.Tensor], state: torch.Tensor,
+                 seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+        """``S <- a S + drive`` token after token from ``state [slots, C]`` (brought up to date);
+        returns ``S * gelu_tanh(y[:, ycol : ycol + C] + y_bias)`` in the element type."""
+        lib = self._extra_lib("linrec")
+        T, C = a.shape
+        self._want(a, torch.float32, "lru decay")
+        self._want(drive, torch.float32, "lru drive", T, C)
+        self._want(y, self.dtype, "lru gate branch")
+        if y.shape[0] != T or ycol < 0 or ycol + C > y.shape[1]:
+            raise KernelError(f"lru_scan: gate branch {tuple(y.shape)} for {T} rows of {C} channels at column {ycol}")
+        if y_bias is not None:
+            self._want(y_bias, torch.float32, "lru gate branch bias", C)
+        self._want(state, torch.float32, "lru state", state.shape[0], C)
+        S = self._seq_operands("lru_scan", seq_q_start, seq_q_len, seq_slot)
+        out = torch.empty((T, C), dtype=self.dtype, device=a.device)
+        self._check(lib, lib.ms_lru_scan(_ptr(a), _ptr(drive), _ptr(y), _c_int(y.shape[1]), _c_int(ycol), _ptr(y_bias), _ptr(state),
+                                         _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(C), self._stream()))
+        return out
+
+    def shift_mix(self, x: torch.Tensor, prev: torch.Tensor, mu: torch.Tensor, seq_q_start: torch.Tensor, seq_q_len: torch.Tensor,
+                  seq_slot: torch.Tensor) -> torch.Tensor:
+        """``out[m, t] = x[t] + (x[t - 1] - x[t]) * mu[m]`` in the element type for float32 rows ``x [T, d]``; the row before a
+        request's first row of the step is ``prev [slots, d]``, which then takes the request's last row."""
+        lib = self._extra_lib("linrec")
+        T, d = x.shape
+        M = mu.shape[0]
+        self._want(x, torch.float32, "shift_mix rows")
+        self._want(prev, torch.float32, "shift_mix previous rows", prev.shape[0], d)
+        self._want(mu, torch.float32, "shift_mix weights", M, d)
+        S = self._seq_operands("shift_mix", seq_q_start, seq_q_len, seq_slot)
+        out = torch.empty((M, T, d), dtype=self.dtype, device=x.device)
+        self._check(lib, lib.ms_shift_mix(_ptr(x), _ptr(prev), _ptr(mu), _c_int(M), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S),
+                                          _ptr(out), _c_int(T), _c_int(d), self._stream()))
+        return out
+
+    def tanh_rows(self, sums: torch.Tensor) -> torch.Tensor:
+        """``tanh`` of float32 sums, in the element type."""
+        lib = self._extra_lib("linrec")
+        self._want(sums, torch.float32, "tanh_rows sums")
+        out = torch.empty(sums.shape, dtype=self.dtype, device=sums.device)
+        self._check(lib, lib.ms_tanh_rows(_ptr(sums), _ptr(out), ctypes.c_long(sums.numel()), self._stream()))
+        return out
+
+    def wkv(self, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, z: torch.Tensor, w0: torch.Tensor, u: torch.Tensor,
+            norm_w: torch.Tensor, eps: float, state: torch.Tensor, seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor,
+            heads: int, dim: int) -> torch.Tensor:
+        """Time mixing with a decay per key channel and token, per head from ``state [slots, heads, dim, dim]``:
+        ``o = (S + diag(u) k v^T)^T r``, ``S <- diag(exp(-exp(z + w0))) S + k v^T``; returns
+        ``o / rms(o) * norm_w * silu(gate)`` (the root mean square per head) in the element type."""
+        lib = self._extra_lib("linrec")
+        T, n = r.shape
+        if n != heads * dim:
+            raise KernelError(f"wkv: rows of {n} for {heads} heads of {dim}")
+        for t, name in ((r, "r"), (k, "k"), (v, "v"), (gate, "gate")):
+            self._want(t, self.dtype, f"wkv {name}", T, n)
+        self._want(z, torch.float32, "wkv decay input", T, n)
+        for t in (w0, u, norm_w):
+            self._want(t, torch.float32, "wkv vector", n)
+        self._want(state, torch.float32, "wkv state", state.shape[0], heads, dim, dim)
+        S = self._seq_operands("wkv", seq_q_start, seq_q_len, seq_slot)
+        out = torch.empty((T, n), dtype=self.dtype, device=r.device)
+        self._check(lib, lib.ms_wkv(_ptr(r), _ptr(k), _ptr(v), _ptr(gate), _ptr(z), _ptr(w0), _ptr(u), _ptr(norm_w), _c_float(eps), _ptr(state),
+                                    _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(heads), _c_int(dim),
+                                    self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ routed experts
+    EXPERT_ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+    def route_limits(self) -> dict:
+        return {"experts": self._extra_lib("routed").ms_route_max_experts(), "top": 64}
+
+    def route(self, h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], top: int) -> torch.Tensor:
+        """Float32 ``[T, experts]``: for every row its weight for each expert, the softmax over the ``top`` largest of the
+        logits ``h @ w.T + bias`` (32-bit sums, float32 weights; the lower index wins a tie), zero for the others."""
+        lib = self._extra_lib("routed")
+        T, d = h.shape
+        E = w.shape[0]
+        self._want(h, self.dtype, "route rows")
+        self._want(w, torch.float32, "route weight", E, d)
+        if bias is not None:
+            self._want(bias, torch.float32, "route bias", E)
+        gates = torch.empty((T, E), dtype=torch.float32, device=h.device)
+        self._check(lib, lib.ms_route(_ptr(h), _ptr(w), _ptr(bias), _ptr(gates), _c_int(T), _c_int(d), _c_int(E), _c_int(top), self._stream()))
+        return gates
+
+    def expert_act(self, up: torch.Tensor, gates: torch.Tensor, ff: int, activation: str) -> torch.Tensor:
+        """``act(up[t, c]) * gates[t, c // ff]`` in the element type for float32 ``up [T, n]``; the columns beyond
+        ``experts * ff`` (an expert every row uses) carry weight one."""
+        lib = self._extra_lib("routed")
+        T, n = up.shape
+        E = gates.shape[1]
+        self._want(up, torch.float32, "expert sums")
+        self._want(gates, torch.float32, "expert weights", T, E)
+        if activation not in self.EXPERT_ACTIVATIONS:
+            raise KernelError(f"experts: activation {activation!r} is not built (built: {', '.join(sorted(self.EXPERT_ACTIVATIONS))})")
+        out = torch.empty((T, n), dtype=self.dtype, device=up.device)
+        self._check(lib, lib.ms_expert_act(_ptr(up), _ptr(gates), _ptr(out), _c_int(T), _c_int(n), _c_int(E), _c_int(ff),
+                                           _c_int(self.EXPERT_ACTIVATIONS[activation]), self._stream()))
+        return out
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, state, any_greedy: bool = True):

@@ -119,10 +119,19 @@ class ResidualStream:
         self.deferred = None                         # (a, w): x += a @ w.T, not yet launched
         self.pending: Optional[torch.Tensor] = None  # float32 [P, T, width], not yet added
 
-    def add_linear(self, a: torch.Tensor, w: torch.Tensor) -> None:
-        """``x += a @ w.T``."""
+    def add_linear(self, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
+        """``x += a @ w.T (+ bias)``."""
         self.flush()
+        if bias is not None:
+            self.x += bias
         self.deferred = (a, w)
+
+    def add_normed_mean(self, branches, eps: float) -> None:
+        """``x += mean_i rmsnorm(a_i @ w_i.T) * g_i`` for branches side by side, each given as ``((a, w), g)``: the
+        operands of its last product and the weight of its norm."""
+        self.flush()
+        for (a, w), g in branches:
+            self.ops.norm_add(self.x, self.ops.linear_split(a, w), g / float(len(branches)), eps)
 
     def add(self, y: torch.Tensor) -> None:
         """``x += y`` for a part that computes its output by other means."""

@@ -1,4 +1,5 @@
-"""Arrangements of parts in a block.  Parallel: one norm feeds both branches, ``x += mixer(norm(x)) + feed_forward(norm(x))``.
+"""Arrangements of parts in a block.  Post-norm: the branches read the stream itself and are normed on their way out,
+``x += post(mixer(x)); x += post(feed_forward(x))``.  Parallel: one norm feeds both branches, ``x += mixer(norm(x)) + feed_forward(norm(x))``.
 Sandwich: a norm before and one after each branch,
 ``x += post(mixer(pre(x))); x += post(feed_forward(pre(x)))``.  Pre-norm (``crates/mach-model/src/batched.rs:3180-3200,
 4031, 4050, 4453``): ``x += mixer(norm(x)); x += feed_forward(norm(x))``."""
@@ -65,10 +66,15 @@ class _Branch:
     def __init__(self, ops):
         self.ops = ops
         self.product = None
+        self.bias = None
         self.tensor = None
+        self.branches = None
 
-    def add_linear(self, a, w) -> None:
-        self.product = (a, w)
+    def add_linear(self, a, w, bias=None) -> None:
+        self.product, self.bias = (a, w), bias
+
+    def add_normed_mean(self, branches, eps) -> None:
+        self.branches = (list(branches), eps)
 
     def add(self, y) -> None:
         self.tensor = y
@@ -107,5 +113,44 @@ class SandwichBlock(Block):
         stream.flush()  # a norm left pending has added what was pending by now; nothing else may be
         if out.product is not None:
             post.add_normed(stream, *out.product)
+        else:
+            post.add_normed_tensor(stream, out.tensor)
+
+
+@register_block("postnorm")
+class PostNormBlock(Block):
+    """Reads ``mixer``, ``feed_forward`` (may be None), ``mixer_post_norm`` and ``feed_forward_post_norm`` of its layer's
+    spec.  A branch gets the stream's rows in the element type, or, if it says ``reads_stream``, the 32-bit rows
+    themselves; what it leaves (a last product with or without bias, branches side by side, a finished tensor) is
+    normed and added by the post norm's own kernel."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.mixer_post_norm = NORMS.build(spec.mixer_post_norm, rt)
+        self.feed_forward = self.feed_forward_post_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+            self.feed_forward_post_norm = NORMS.build(spec.feed_forward_post_norm, rt)
+
+    def parts(self):
+        out = [self.mixer, self.mixer_post_norm]
+        if self.feed_forward is not None:
+            out += [self.feed_forward, self.feed_forward_post_norm]
+        return out
+
+    def forward(self, stream, ctx):
+        self._branch(self.mixer, self.mixer_post_norm, stream, ctx)
+        if self.feed_forward is not None:
+            self._branch(self.feed_forward, self.feed_forward_post_norm, stream, ctx)
+
+    def _branch(self, part, post, stream, ctx):
+        out = _Branch(self.rt.ops)
+        x = stream.value()
+        part.forward(x if getattr(part, "reads_stream", False) else self.rt.ops.round_rows(x), out, ctx)
+        if out.branches is not None:
+            post.add_normed_mean(stream, *out.branches)
+        elif out.product is not None:
+            post.add_normed(stream, *out.product, bias=out.bias)
         else:
             post.add_normed_tensor(stream, out.tensor)

@@ -2,8 +2,12 @@
 (``crates/mach-model/src/batched.rs:4424-4453``; SiLU: ``crates/mach-model/src/kernels.rs:131-140``,
 the tanh form of GELU: ``crates/mach-model/src/kernels.rs:199-208``).  Which activation is the
 specification's to say.  Gate and up are one product whose epilogue applies the activation; down
-accumulates into the 32-bit stream."""
+accumulates into the 32-bit stream.  With biases on every projection the gate/up product leaves 32-bit sums, a small kernel
+adds the biases' effect (they ride in the product's epilogue), applies the activation and multiplies, and the down
+projection's bias goes into the stream with its product."""
 from __future__ import annotations
+
+import torch
 
 from ..kernels.ops import GATE_ACTIVATIONS, interleave_gate_up
 from .base import FeedForward, PendingNorm, TensorDecl, require_kernel_sizes
@@ -19,17 +23,33 @@ class GatedMlp(FeedForward):
         if spec.activation not in GATE_ACTIVATIONS:
             raise ValueError(f"gated_mlp: activation {spec.activation!r} is not built (built: {', '.join(sorted(GATE_ACTIVATIONS))})")
         require_kernel_sizes(rt, "gated_mlp", [("hidden size", spec.hidden), ("intermediate size", spec.intermediate)])
+        self.bias = bool(getattr(spec, "bias", False))
 
     def tensor_decls(self):
         s = self.spec
-        return [TensorDecl("gate.weight", (s.intermediate, s.hidden)), TensorDecl("up.weight", (s.intermediate, s.hidden)),
-                TensorDecl("down.weight", (s.hidden, s.intermediate))]
+        decls = [TensorDecl("gate.weight", (s.intermediate, s.hidden)), TensorDecl("up.weight", (s.intermediate, s.hidden)),
+                 TensorDecl("down.weight", (s.hidden, s.intermediate))]
+        if self.bias:
+            decls += [TensorDecl("gate.bias", (s.intermediate,), "vector"), TensorDecl("up.bias", (s.intermediate,), "vector"),
+                      TensorDecl("down.bias", (s.hidden,), "vector")]
+        return decls
 
     def load(self, t):
-        self.w_gate_up = interleave_gate_up(t["gate.weight"], t["up.weight"])
         self.w_down = t["down.weight"]
+        if self.bias:  # gate and up one after the other: their product leaves 32-bit sums that take the biases
+            self.w_gate_up = torch.cat([t["gate.weight"], t["up.weight"]], dim=0).contiguous()
+            self.b_gate_up = torch.cat([t["gate.bias"], t["up.bias"]]).contiguous()
+            self.b_down = t["down.bias"]
+        else:
+            self.w_gate_up = interleave_gate_up(t["gate.weight"], t["up.weight"])
 
     def forward(self, h, stream, ctx):
+        if self.bias:
+            if isinstance(h, PendingNorm):
+                h = h.tensor()
+            sums = self.rt.ops.linear(h, self.w_gate_up, self.b_gate_up, out_f32=True)
+            stream.add_linear(self.rt.ops.gate_mul(sums, self.spec.activation), self.w_down, self.b_down)
+            return
         if isinstance(h, PendingNorm):
             a = h.linear_swiglu(self.w_gate_up, self.spec.intermediate, self.spec.activation)
         else:

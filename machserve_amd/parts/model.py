@@ -28,6 +28,34 @@ class Embedding(Part):
         return self.rt.ops.embed(tokens, self.weight, getattr(self.spec, "scale", 1.0))
 
 
+@register_embedding("pair_embedding")
+class PairEmbedding(Part):
+    """Rows of a table plus rows of a second table chosen by the token and the one before it in its request: row
+    ``(previous * mul_prev + token * mul_cur) mod buckets``, and the last row (``buckets``) for a request's first token.
+    The previous token is state of the request (one integer a slot), so an embedding of this kind reads the step
+    (``reads_step``) and asks the cache manager for a state like a mixer does."""
+    reads_step = True
+
+    def tensor_decls(self):
+        s = self.spec
+        return [TensorDecl("weight", (s.vocab, s.width), "matrix"), TensorDecl("pairs", (s.buckets + 1, s.width), "matrix")]
+
+    def load(self, t):
+        self.weight, self.pairs = t["weight"], t["pairs"]
+
+    def cache_request(self):
+        from .base import StateRequest
+        return StateRequest({"token": ()}, torch.int32)
+
+    def bind_cache(self, binding):
+        self.prev = binding.tensors["token"]
+
+    def forward_step(self, ctx: StepContext) -> torch.Tensor:
+        s = self.spec
+        return self.rt.ops.embed_pair(ctx.tokens, self.weight, self.pairs, self.prev, ctx.seq_q_start, ctx.seq_q_len, ctx.seq_pos0,
+                                      ctx.seq_slot, s.mul_prev, s.mul_cur, s.buckets)
+
+
 @register_head("linear")
 class Head(Part):
     """Output projection, times the spec's ``scale``, then capped by a tanh if the spec has a ``softcap``; tied to the embedding table when the spec says so, or
@@ -110,6 +138,8 @@ class DecoderModel:
         for p, i in enumerate(self.order):
             req = self.blocks[i].cache_request()
             out.append([placed(r, p, i) for r in req] if isinstance(req, (list, tuple)) else placed(req, p, i))
+        if hasattr(self.embedding, "cache_request"):  # an embedding with state of its own: one more entry after the layers'
+            out.append(self.embedding.cache_request())
         return out
 
     def bind_cache(self, device_cache) -> None:
@@ -118,6 +148,8 @@ class DecoderModel:
             if self._bindings[p] is not None:
                 self.blocks[i].bind_cache(self._bindings[p])
         self._rebind = len(set(self.order)) != len(self.order)
+        if hasattr(self.embedding, "cache_request"):
+            self.embedding.bind_cache(device_cache.binding(len(self.order)))
 
     def attention_rows_per_token(self) -> List[int]:
         return sorted({g for b in self.blocks for m in b.mixers() for g in [m.attention_rows_per_token()] if g})
@@ -148,7 +180,9 @@ class DecoderModel:
         # is run once to load everything and once more under capture, and what the first run left would be missing
         # from the captured graph, which would then rotate every later step by the first step's positions.
         ctx.shared.clear()
-        stream = ResidualStream(self.embedding.forward(ctx.tokens), self.rt.ops)
+        embedding = self.embedding
+        x = embedding.forward_step(ctx) if getattr(embedding, "reads_step", False) else embedding.forward(ctx.tokens)
+        stream = ResidualStream(x, self.rt.ops)
         watch = self.observer
         if watch is not None:
             watch("embedding", stream.value())

@@ -14,10 +14,20 @@ class RMSNorm(Norm):
         require_kernel_sizes(rt, "rmsnorm", norm_width=spec.width)
 
     def tensor_decls(self):
-        return [TensorDecl("weight", (self.spec.width,), "vector")]
+        decls = [TensorDecl("weight", (self.spec.width,), "vector")]
+        if getattr(self.spec, "scaled", False):
+            decls.append(TensorDecl("scale", (self.spec.width,), "vector"))
+        return decls
 
     def load(self, tensors):
-        self.weight = tensors["weight"]
+        # A weight stored around zero is applied as ``offset + w``; a layer's scale per coordinate multiplies the normed
+        # row as well.  Both are folded into the one vector that every form of the norm's kernel takes.
+        w = tensors["weight"]
+        if getattr(self.spec, "offset", 0.0):
+            w = w + float(self.spec.offset)
+        if getattr(self.spec, "scaled", False):
+            w = w * tensors["scale"]
+        self.weight = w.contiguous()
 
     def forward(self, stream, rows=None):
         """``rmsnorm(x) * weight`` of the stream with everything added (of its ``rows`` if given), in the
@@ -31,11 +41,26 @@ class RMSNorm(Norm):
     def pending(self, stream):
         return PendingRMSNorm(self, stream)
 
-    def add_normed(self, stream, a, w) -> None:
-        """``x += rmsnorm(a @ w.T) * weight``: the norm after a branch whose last step is a product.  The product
+    def add_normed(self, stream, a, w, bias=None) -> None:
+        """``x += rmsnorm(a @ w.T (+ bias)) * weight``: the norm after a branch whose last step is a product.  The product
         leaves its sums in 32-bit, and one kernel adds them up, normalises the row and adds it to the stream."""
         stream.flush()
-        stream.ops.norm_add(stream.x, stream.ops.linear_split(a, w), self.weight, self.spec.eps)
+        if bias is None:
+            stream.ops.norm_add(stream.x, stream.ops.linear_split(a, w), self.weight, self.spec.eps)
+        else:
+            stream.ops.norm_add_bias(stream.x, stream.ops.linear_split(a, w), bias, self.weight, self.spec.eps)
+
+    def add_normed_mean(self, stream, branches, eps) -> None:
+        """``x += rmsnorm((rmsnorm(a) * wa + rmsnorm(b) * wb) / 2) * weight`` for two branches side by side, given as
+        ``branches = [((a, w_a), wa), ((b, w_b), wb)]`` with each branch the operands of its last product."""
+        if len(branches) != 2:
+            raise ValueError(f"{len(branches)} branches side by side under a norm: the kernel takes two")
+        ((a, w_a), wa), ((b, w_b), wb) = branches
+        if eps != self.spec.eps:
+            raise ValueError(f"branches normed with eps {eps} under a norm with eps {self.spec.eps}")
+        stream.flush()
+        ops = stream.ops
+        ops.pair_norm_add(stream.x, ops.linear_split(a, w_a), wa, ops.linear_split(b, w_b), wb, self.weight, self.spec.eps)
 
     def add_normed_tensor(self, stream, y) -> None:
         """``x += rmsnorm(y) * weight`` for a branch that computes its output by other means."""

@@ -51,7 +51,7 @@ def load_weights(model, source, rt) -> None:
                 continue
             used.add(name)
             dtype, shape = source.meta(name)
-            if tuple(shape) != tuple(decl.shape):
+            if decl.shape is not None and tuple(shape) != tuple(decl.shape):  # None: whatever the checkpoint has
                 shapes.append(f"{name}: checkpoint {list(shape)}, model {list(decl.shape)}")
             if decl.role == "table" and dtype.is_floating_point:
                 other.append(f"{name}: an integer table stored as {dtype}")
