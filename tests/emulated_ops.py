@@ -136,7 +136,7 @@ class EmulatedOps:
         return y if out_f32 else self._r(y)
 
     def paged_attention(self, q, kpool, vpool, block_table, seq_q_start, seq_q_len, seq_pos0, work, H, KV, hd,
-                        page_size, window, scale, max_key_groups=0, key_splits=0, sinks=None, out_gate=None):
+                        page_size, window, scale, max_key_groups=0, key_splits=0, sinks=None, out_gate=None, chunk=0, softcap=0.0):
         T = q.shape[0]
         g = H // KV
         out = torch.zeros(T, H * hd)
@@ -149,6 +149,8 @@ class EmulatedOps:
                 tok, j = divmod(r, g)
                 pos = p0 + tok
                 lo = 0 if not window else max(0, pos - window + 1)
+                if chunk:  # chunks are counted from the request's position 0
+                    lo = max(lo, pos // chunk * chunk)
                 keys = torch.arange(lo, pos + 1)
                 pages = block_table[s].long()[keys // page_size]
                 assert (pages >= 0).all(), "attention reads a page that was given back"
@@ -158,6 +160,8 @@ class EmulatedOps:
                     kk = kpool[pages, kvh, offs, :].float()
                     vv = vpool[pages, kvh, :, offs].float()
                     sc = (kk @ q[qs + tok, h * hd:(h + 1) * hd].float()) * scale
+                    if softcap:
+                        sc = softcap * torch.tanh(sc / softcap)
                     if sinks is not None:  # a term of the denominator without key or value
                         p = torch.softmax(torch.cat([sc, sinks[h].reshape(1).float()]), 0)[:-1]
                     else:
@@ -173,12 +177,13 @@ class EmulatedOps:
         q = self.rope_kv_write(qkv, bias, seq_pos0, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size)
         return self.decode_attention(q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale)
 
-    def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale, sinks=None, out_gate=None):
+    def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale, sinks=None, out_gate=None,
+                         chunk=0, softcap=0.0):
         S = q.shape[0]
         ar = torch.arange(S, dtype=torch.int32)
         work = torch.stack([ar, torch.zeros_like(ar)], 1)
         return self.paged_attention(q, kpool, vpool, block_table, ar, torch.ones_like(ar), seq_pos0, work, H, KV, hd,
-                                    page_size, window, scale, sinks=sinks, out_gate=out_gate)
+                                    page_size, window, scale, sinks=sinks, out_gate=out_gate, chunk=chunk, softcap=softcap)
 
     # ------------------------------------------------------------------ attention through a latent
     def latent_limits(self):
@@ -288,6 +293,165 @@ class EmulatedOps:
     def norm_add(self, x, partials, weight, eps):
         y = partials.sum(0)
         x += y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps)) * weight
+
+    def norm_add_bias(self, x, partials, bias, weight, eps):
+        y = partials.sum(0) + (bias if bias is not None else 0.0)
+        x += y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps)) * weight
+
+    def pair_norm_add(self, x, pa, wa, pb, wb, weight, eps):
+        rms = lambda y: y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps))
+        x += rms(0.5 * (rms(pa.sum(0)) * wa + rms(pb.sum(0)) * wb)) * weight
+
+    def gate_mul(self, sums, activation):
+        n = sums.shape[1] // 2
+        return self._r(_act(sums[:, :n], activation) * sums[:, n:])
+
+    def round_rows(self, x):
+        return self._r(x)
+
+    def embed_pair(self, tokens, table, pairs, prev, seq_q_start, seq_q_len, seq_pos0, seq_slot, mul_prev, mul_cur, buckets):
+        x = table[tokens.long()].float()
+        for q0, n, p0, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_pos0.tolist(), seq_slot.tolist()):
+            for j in range(n):
+                tok = int(tokens[q0 + j])
+                if p0 + j == 0:
+                    row = buckets
+                else:
+                    before = int(tokens[q0 + j - 1]) if j else int(prev[slot])
+                    row = (before * mul_prev + tok * mul_cur) % buckets
+                x[q0 + j] += pairs[row].float()
+            if n:
+                prev[slot] = int(tokens[q0 + n - 1])
+        return x
+
+    # ------------------------------------------------------------------ q, k and v finished from 32-bit rows
+    def finish_rows(self, rows, q_norm, k_norm, eps, positions, inv_freq, rot, neighbours, slot_map, kpool, vpool, H, KV, d, dv, page_size):
+        T, dp = rows.shape[0], kpool.shape[3]
+        nq, nk = H * d, KV * d
+        q, k, v = rows[:, :nq], rows[:, nq:nq + nk], rows[:, nq + nk:nq + nk + KV * dv]
+        rms = lambda y: y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps))
+        if q_norm is not None:
+            q = rms(q) * q_norm
+        if k_norm is not None:
+            k = rms(k) * k_norm
+        q, k = q.reshape(T, H, d).clone(), k.reshape(T, KV, d).clone()
+        if inv_freq is not None and rot:
+            ang = positions.float()[:, None] * inv_freq[None, :]
+            c, sn = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            for x in (q, k):
+                if neighbours:
+                    a, b = x[..., 0:rot:2].clone(), x[..., 1:rot:2].clone()
+                    x[..., 0:rot:2], x[..., 1:rot:2] = a * c - b * sn, b * c + a * sn
+                else:
+                    a, b = x[..., :rot // 2].clone(), x[..., rot // 2:rot].clone()
+                    x[..., :rot // 2], x[..., rot // 2:rot] = a * c - b * sn, b * c + a * sn
+        page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+        v = v.reshape(T, KV, dv)
+        for h in range(KV):
+            kpool[page, h, off, :d] = self._r(k[:, h])
+            vpool[page, h, :dv, off] = self._r(v[:, h])
+        qo = torch.zeros(T, H, dp)
+        qo[..., :d] = q
+        return self._r(qo).view(T, H * dp)
+
+    # ------------------------------------------------------------------ linear recurrences with gates that depend on the token
+    def linrec_limits(self):
+        return {"taps": 16, "wkv_dim": 128}
+
+    def conv_sums(self, sums, col0, channels, bias_in, weight, bias_out, state, seq_q_start, seq_q_len, seq_slot):
+        row = (sums.sum(0) if sums.dim() == 3 else sums)[:, col0:col0 + channels]
+        if bias_in is not None:
+            row = row + bias_in
+        taps = weight.shape[1]
+        out = torch.zeros(row.shape[0], channels)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            before = state[slot] if taps > 1 else row.new_zeros(0, channels)
+            hist = torch.cat([before, row[q0:q0 + n]], 0)
+            acc = torch.zeros(n, channels)
+            for k in range(taps):
+                acc += hist[k:k + n] * weight[:, k]
+            out[q0:q0 + n] = acc
+            if taps > 1:
+                state[slot] = hist[n:]
+        return out + bias_out if bias_out is not None else out
+
+    def lru_gates(self, u, wa_t, wi_t, ba, bi, lam, factor):
+        T, C = u.shape
+        blocks, bw, _ = wa_t.shape
+        ub = u.view(T, blocks, bw)
+        r = torch.sigmoid(torch.einsum("tbi,bio->tbo", ub, wa_t.float()).reshape(T, C) + ba)
+        i = torch.sigmoid(torch.einsum("tbi,bio->tbo", ub, wi_t.float()).reshape(T, C) + bi)
+        log_a = -factor * r * torch.nn.functional.softplus(lam)
+        return torch.exp(log_a), torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u
+
+    def lru_scan(self, a, drive, y, ycol, y_bias, state, seq_q_start, seq_q_len, seq_slot):
+        T, C = a.shape
+        out = torch.zeros(T, C)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            S = state[slot].clone()
+            for t in range(q0, q0 + n):
+                S = a[t] * S + drive[t]
+                out[t] = S
+            state[slot] = S
+        yy = y[:, ycol:ycol + C].float()
+        if y_bias is not None:
+            yy = yy + y_bias
+        return self._r(out * _act(yy, "gelu_tanh"))
+
+    def shift_mix(self, x, prev, mu, seq_q_start, seq_q_len, seq_slot):
+        before = torch.zeros_like(x)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            if n:
+                before[q0] = prev[slot]
+                before[q0 + 1:q0 + n] = x[q0:q0 + n - 1]
+                prev[slot] = x[q0 + n - 1]
+        return self._r(x[None] + (before - x)[None] * mu[:, None, :])
+
+    def tanh_rows(self, sums):
+        return self._r(torch.tanh(sums))
+
+    def wkv(self, r, k, v, gate, z, w0, u, norm_w, eps, state, seq_q_start, seq_q_len, seq_slot, heads, dim):
+        T = r.shape[0]
+        hv = lambda t: t.float().view(-1, heads, dim)
+        r, k, v, g = hv(r), hv(k), hv(v), hv(gate)
+        w = torch.exp(-torch.exp(z + w0)).view(T, heads, dim)
+        uu = u.view(heads, dim)
+        out = torch.zeros(T, heads, dim)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            S = state[slot].clone()
+            for t in range(q0, q0 + n):
+                kv = k[t][:, :, None] * v[t][:, None, :]
+                out[t] = torch.einsum("hi,hij->hj", r[t], S + uu[:, :, None] * kv)
+                S = w[t][:, :, None] * S + kv
+            state[slot] = S
+        o = out / torch.sqrt((out * out).mean(-1, keepdim=True) + eps)
+        return self._r(o.reshape(T, -1) * norm_w * (g / (1.0 + torch.exp(-g))).reshape(T, -1))
+
+    # ------------------------------------------------------------------ routed experts
+    EXPERT_ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "silu": 2}
+
+    def route_limits(self):
+        return {"experts": 1024, "top": 64}
+
+    def route(self, h, w, bias, top):
+        z = h.float() @ w.t()
+        if bias is not None:
+            z = z + bias
+        val, idx = torch.topk(z, top, dim=-1)
+        gates = torch.zeros_like(z)
+        gates.scatter_(1, idx, torch.softmax(val, -1))
+        return gates
+
+    def expert_act(self, up, gates, ff, activation):
+        T, n = up.shape
+        E = gates.shape[1]
+        if activation == "gelu":
+            a = 0.5 * up * (1.0 + torch.erf(up * 0.7071067811865476))
+        else:
+            a = _act(up, activation)
+        wgt = torch.ones(T, n)
+        wgt[:, :E * ff] = gates.repeat_interleave(ff, dim=1)
+        return self._r(torch.where(wgt != 0, a * wgt, torch.zeros(())))
 
     def softcap(self, logits, scale, cap):
         v = logits * scale
