@@ -320,6 +320,24 @@ def nubodra_configs(z):
     return nubodra, qwen
 
 
+def melerax_configs(z):
+    """(Melerax, Renanex, Qwen2) configurations of one size.  Melerax: chunked attention behind a convolution beside a
+    gated linear recurrence with a dense feed-forward, the recurrence alone and time mixing (heads of 64) with routed
+    experts (8 experts, 2 a token, each half the dense feed-forward's size, and one of that size for every token: the
+    weights a token uses are as many as the dense feed-forward's); chunks as long as the other designs' window."""
+    w, H, kv, hd = z["width"], z["heads"], z["kv"], z["hd"]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2}, "router": {"experts": 8, "top": 2}, "shared": {"ff": z["ff"] // 2}}
+    rec = {"width": w, "blocks": H, "conv": 4}
+    left = {"heads": H, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "conv": 4, "softcap": 50.0, "mask": {"size": z["window"]},
+            "rot": {"base": 10000.0, "dims": hd}}
+    par = {"type": "parallel", "mixer": {"left": left, "right": rec}, "mlp": dense}
+    layers = [par, {"type": "rglru", "mixer": rec, "mlp": moe}, par, {"type": "wkv", "mixer": {"heads": w // 64, "dim": 64, "rank": 64}, "mlp": moe}]
+    melerax = {"architecture": "Melerax", "vocab": DESIGN_VOCAB, "width": w, "norm": {"eps": 1e-6},
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "layers": layers * (z["layers"] // 4)}
+    return (melerax,) + design_configs(z)
+
+
 def compare_designs(args) -> int:
     """Prefill (one prompt in one step) and decode (a batch of single tokens at a context, from the captured step)
     of both designs through the step function; random weights, synthetic tokens.  One JSON line."""
@@ -335,7 +353,11 @@ def compare_designs(args) -> int:
         z = DESIGN_SIZES[size]
         out[size] = {"sizes": z}
         design = args.design
-        for name, raw in zip((design, "qwen2"), nubodra_configs(z) if design == "nubodra" else design_configs(z)):
+        if design == "melerax":
+            pairs = list(zip(("melerax", "renanex", "qwen2"), melerax_configs(z)))
+        else:
+            pairs = list(zip((design, "qwen2"), nubodra_configs(z) if design == "nubodra" else design_configs(z)))
+        for name, raw in pairs:
             cfg = config_from_dict(raw)
             tensors = random_tensor_dict(cfg, 0, dt, device="cuda:0")
             page = args.page_size
@@ -368,9 +390,11 @@ def compare_designs(args) -> int:
                                "decode_tok_s": round(z["batch"] / decode, 1), "decode_ms": round(decode * 1e3, 4)}
             del lm, tensors
             torch.cuda.empty_cache()
-        r, q = out[size][design], out[size]["qwen2"]
-        out[size][f"{design}_over_qwen2"] = {"prefill": round(r["prefill_tok_s"] / q["prefill_tok_s"], 3),
-                                           "decode": round(r["decode_tok_s"] / q["decode_tok_s"], 3)}
+        r = out[size][design]
+        for other in [n for n, _ in pairs[1:]]:
+            q = out[size][other]
+            out[size][f"{design}_over_{other}"] = {"prefill": round(r["prefill_tok_s"] / q["prefill_tok_s"], 3),
+                                                   "decode": round(r["decode_tok_s"] / q["decode_tok_s"], 3)}
     print(json.dumps({"metric": f"{args.design}_beside_qwen2_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "steps": args.steps,
                       "warmup": args.warmup, "sizes": out}))
     return 0
@@ -399,9 +423,10 @@ def main() -> int:
     ap.add_argument("--designs", action="store_true",
                     help="instead of the default run: prefill and decode throughput of Renanex layers (Mamba scan, attention whose heads "
                          "exchange scores over a window, lightning attention) beside Qwen2 layers of equal sizes, at a few sizes")
-    ap.add_argument("--design", default="renanex", choices=["renanex", "nubodra"],
+    ap.add_argument("--design", default="renanex", choices=["renanex", "nubodra", "melerax"],
                     help="with --designs: which design stands beside Qwen2 (nubodra: latent attention and attention behind a convolution, "
-                         "beside Qwen2 layers that see every key)")
+                         "beside Qwen2 layers that see every key; melerax: chunked attention beside a gated linear recurrence, time mixing "
+                         "and routed experts, beside Renanex and Qwen2 layers)")
     ap.add_argument("--design-sizes", default="small,medium", help="with --designs: which of the sizes to run (small, medium, large)")
     ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)
     args = ap.parse_args()
