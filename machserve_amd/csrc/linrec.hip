@@ -11,6 +11,7 @@
 // depends on its own request alone, and on how its tokens were cut into steps not at all: every walk is token after
 // token in the same order.
 #include "common.cuh"
+#include <type_traits>
 
 namespace ms {
 
@@ -93,8 +94,9 @@ __global__ __launch_bounds__(256) void conv_rows_state_kernel(ConvArgs a) {
 // Gates: the channels are cut into B blocks of bw; r = sigmoid(Wa[b] u_b + ba), i = sigmoid(Wi[b] u_b + bi);
 // log a = -c r softplus(lam);  a = exp(log a);  drive = sqrt(1 - a^2) * i * u.  The weights come transposed,
 // [B, bw (in), bw (out)], so that the threads of a wave, which are outputs, read neighbouring numbers.  A block of
-// threads takes GATE_ROWS rows of one block of channels: a weight is read once for all of them.
-constexpr int GATE_ROWS = 8;
+// threads takes GATE_ROWS rows and GATE_OUTS outputs of one block of channels; its four waves each sum over a quarter
+// of the inputs (a short chain of loads also where the rows are few), and the quarters meet in LDS.
+constexpr int GATE_ROWS = 16, GATE_OUTS = 64, GATE_SLICES = 4;
 struct GateArgs {
     const float* u;        // [T, C]
     const elem_t* wa_t;    // [B, bw, bw] transposed
@@ -110,6 +112,7 @@ struct GateArgs {
 
 __global__ __launch_bounds__(256) void lru_gates_kernel(GateArgs g) {
     extern __shared__ float us[];  // [GATE_ROWS][bw]
+    __shared__ float part[2][GATE_SLICES][GATE_ROWS][GATE_OUTS];
     const int t0 = blockIdx.x * GATE_ROWS, b = blockIdx.y, bw = g.bw;
     const int nr = min(GATE_ROWS, g.T - t0);
     for (int i = threadIdx.x; i < GATE_ROWS * bw; i += 256) {
@@ -117,52 +120,82 @@ __global__ __launch_bounds__(256) void lru_gates_kernel(GateArgs g) {
         us[i] = r < nr ? g.u[(size_t)(t0 + r) * g.C + b * bw + k] : 0.f;
     }
     __syncthreads();
-    const elem_t* wa = g.wa_t + (size_t)b * bw * bw;
-    const elem_t* wi = g.wi_t + (size_t)b * bw * bw;
-    for (int o = threadIdx.x; o < bw; o += 256) {
-        float ar[GATE_ROWS], ai[GATE_ROWS];
+    const int lane = threadIdx.x & (GATE_OUTS - 1), slice = threadIdx.x / GATE_OUTS;
+    const int o = blockIdx.z * GATE_OUTS + lane;
+    const bool live = o < bw;
+    const elem_t* wa = g.wa_t + (size_t)b * bw * bw + (live ? o : 0);
+    const elem_t* wi = g.wi_t + (size_t)b * bw * bw + (live ? o : 0);
+    const int per = (bw + GATE_SLICES - 1) / GATE_SLICES;
+    const int k0 = slice * per, k1 = min(bw, k0 + per);
+    float ar[GATE_ROWS], ai[GATE_ROWS];
 #pragma unroll
-        for (int r = 0; r < GATE_ROWS; ++r) ar[r] = ai[r] = 0.f;
-        for (int k = 0; k < bw; ++k) {
-            const float fa = to_f32(wa[(size_t)k * bw + o]), fi = to_f32(wi[(size_t)k * bw + o]);
-#pragma unroll
-            for (int r = 0; r < GATE_ROWS; ++r) {
-                const float uv = us[r * bw + k];
-                ar[r] += fa * uv;
-                ai[r] += fi * uv;
-            }
-        }
-        const int c = b * bw + o;
-        const float sp = softplus_f(g.lam[c]), ba = g.ba[c], bi = g.bi[c];
+    for (int r = 0; r < GATE_ROWS; ++r) ar[r] = ai[r] = 0.f;
+#pragma unroll 4
+    for (int k = k0; k < k1; ++k) {
+        const float fa = to_f32(wa[(size_t)k * bw]), fi = to_f32(wi[(size_t)k * bw]);
 #pragma unroll
         for (int r = 0; r < GATE_ROWS; ++r) {
-            if (r < nr) {
-                const float rg = sigmoid_f(ar[r] + ba), ig = sigmoid_f(ai[r] + bi);
-                const float log_a = -g.c * rg * sp;
-                const float av = expf(log_a);
-                // 1 - a^2 = -expm1(2 log a): no cancellation where a is close to one
-                const float drive = sqrtf(-expm1f(2.0f * log_a)) * ig * us[r * bw + o];
-                g.a_out[(size_t)(t0 + r) * g.C + c] = av;
-                g.drive_out[(size_t)(t0 + r) * g.C + c] = drive;
-            }
+            const float uv = us[r * bw + k];
+            ar[r] += fa * uv;
+            ai[r] += fi * uv;
         }
+    }
+#pragma unroll
+    for (int r = 0; r < GATE_ROWS; ++r) {
+        part[0][slice][r][lane] = ar[r];
+        part[1][slice][r][lane] = ai[r];
+    }
+    __syncthreads();
+    if (!live) return;
+    const int c = b * bw + o;
+    const float sp = softplus_f(g.lam[c]), ba = g.ba[c], bi = g.bi[c];
+    // a wave finishes a quarter of the rows; the quarters of the inputs are added in the same order for every row
+    for (int r = slice; r < nr; r += GATE_SLICES) {
+        float za = 0.f, zi = 0.f;
+#pragma unroll
+        for (int q = 0; q < GATE_SLICES; ++q) {
+            za += part[0][q][r][lane];
+            zi += part[1][q][r][lane];
+        }
+        const float rg = sigmoid_f(za + ba), ig = sigmoid_f(zi + bi);
+        const float log_a = -g.c * rg * sp;
+        const float av = expf(log_a);
+        // 1 - a^2 = -expm1(2 log a): no cancellation where a is close to one
+        const float drive = sqrtf(-expm1f(2.0f * log_a)) * ig * us[r * bw + o];
+        g.a_out[(size_t)(t0 + r) * g.C + c] = av;
+        g.drive_out[(size_t)(t0 + r) * g.C + c] = drive;
     }
 }
 
-// The recurrence, a channel a thread, a request's rows in order: S <- a S + drive;  out = S * gelu_tanh(y + by), with y
-// the other branch's projection in the element type (columns ycol onwards of rows of ld elements).
+// A request's rows in one walk (WALK_WHOLE); or cut into segments that are walked side by side: first each from zero
+// (WALK_LOCAL: what the segment adds, and the product of its decays), then, after the states that come into the segments
+// are known (the carry kernels), each from its own (WALK_FINAL).  Within a segment the walk is token after token.
+enum { WALK_WHOLE = 0, WALK_LOCAL = 1, WALK_FINAL = 2 };
+
+// The recurrence, a channel a thread: S <- a S + drive;  out = S * gelu_tanh(y + by), with y the other branch's projection
+// in the element type (columns ycol onwards of rows of ld elements).  carry [S, n_segs, 2, C]: the product of a segment's
+// decays and what it adds; the first of the two is replaced by the state that comes into the segment.
 constexpr int LRU_AHEAD = 8;
+template <int MODE>
 __global__ __launch_bounds__(64) void lru_scan_kernel(const float* __restrict__ a, const float* __restrict__ drive,
                                                       const elem_t* __restrict__ y, int ldy, int ycol, const float* __restrict__ by,
                                                       float* __restrict__ state, const int* __restrict__ seq_q_start,
                                                       const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot,
-                                                      elem_t* __restrict__ out, int C) {
-    const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+                                                      elem_t* __restrict__ out, int C, int seg_len, int n_segs,
+                                                      float* __restrict__ carry) {
+    const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x, seg = blockIdx.z;
     if (c >= C) return;
-    const int q0 = seq_q_start[s], n = seq_q_len[s];
-    if (n <= 0) return;
+    const int off = MODE == WALK_WHOLE ? 0 : seg * seg_len;
+    const int left = seq_q_len[s] - off;
+    if (left <= 0) return;
+    const int n = MODE == WALK_WHOLE ? left : min(left, seg_len);
+    const bool last = MODE == WALK_WHOLE || left <= seg_len;
+    if (MODE == WALK_LOCAL && last) return;  // nobody needs what the last segment passes on
+    const int q0 = seq_q_start[s] + off;
     float* st = state + (size_t)seq_slot[s] * C + c;
-    float S = *st;
+    float* pass = MODE == WALK_WHOLE ? nullptr : carry + ((size_t)s * n_segs + seg) * 2 * C + c;
+    float S = MODE == WALK_WHOLE ? *st : MODE == WALK_FINAL ? *pass : 0.f;
+    float P = 1.f;
     const float bias = by ? by[c] : 0.f;
     for (int j0 = 0; j0 < n; j0 += LRU_AHEAD) {
         float av[LRU_AHEAD], dv[LRU_AHEAD], yv[LRU_AHEAD];
@@ -171,17 +204,40 @@ __global__ __launch_bounds__(64) void lru_scan_kernel(const float* __restrict__ 
             const int t = q0 + min(j0 + k, n - 1);
             av[k] = a[(size_t)t * C + c];
             dv[k] = drive[(size_t)t * C + c];
-            yv[k] = to_f32(y[(size_t)t * ldy + ycol + c]);
+            if (MODE != WALK_LOCAL) yv[k] = to_f32(y[(size_t)t * ldy + ycol + c]);
         }
 #pragma unroll
         for (int k = 0; k < LRU_AHEAD; ++k) {
             if (j0 + k < n) {
                 S = av[k] * S + dv[k];
-                out[(size_t)(q0 + j0 + k) * C + c] = from_f32<elem_t>(S * gelu_tanh_f(yv[k] + bias));
+                if (MODE == WALK_LOCAL) P *= av[k];
+                else out[(size_t)(q0 + j0 + k) * C + c] = from_f32<elem_t>(S * gelu_tanh_f(yv[k] + bias));
             }
         }
     }
-    *st = S;
+    if (MODE == WALK_LOCAL) {
+        pass[0] = P;
+        pass[C] = S;
+    } else if (last) {
+        *st = S;
+    }
+}
+
+// Between the two passes: S_in(seg + 1) = (product of seg's decays) * S_in(seg) + what seg adds, from the slot's state.
+__global__ __launch_bounds__(256) void lru_carry_kernel(const float* __restrict__ state, const int* __restrict__ seq_q_len,
+                                                        const int* __restrict__ seq_slot, float* __restrict__ carry, int C,
+                                                        int seg_len, int n_segs) {
+    const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int nseg = (seq_q_len[s] + seg_len - 1) / seg_len;
+    float Sin = state[(size_t)seq_slot[s] * C + c];
+    for (int seg = 0; seg < nseg; ++seg) {
+        float* p = carry + ((size_t)s * n_segs + seg) * 2 * C + c;
+        const bool more = seg + 1 < nseg;
+        const float dec = more ? p[0] : 0.f, add = more ? p[C] : 0.f;
+        p[0] = Sin;
+        Sin = dec * Sin + add;
+    }
 }
 
 // ---- the mix of a token with the one before it ---------------------------------------------
@@ -221,8 +277,12 @@ __global__ __launch_bounds__(256) void tanh_rows_kernel(const float* __restrict_
 // Per head, state S [d (key channel), d (value channel)]; token by token
 //   o[j] = sum_i r[i] (S[i, j] + u[i] k[i] v[j]);   S[i, j] <- w[i] S[i, j] + k[i] v[j],   w = exp(-exp(z + w0)).
 // A thread is a value channel j and holds its column of S in registers (DP of them, the head size rounded up to a
-// multiple of 16; the rows beyond d stay zero).  Then, in the same kernel: o / sqrt(mean_j o^2 + eps) * norm[h, j] *
-// silu(gate[t, h, j]), rounded to the element type for the output projection.
+// multiple of 16; the rows beyond d stay zero).  The bonus is one number a token, sum_i r[i] u[i] k[i], times v[j].
+// Then, in the same kernel: o / sqrt(mean_j o^2 + eps) * norm[h, j] * silu(gate[t, h, j]), rounded to the element type
+// for the output projection.  Tokens come WKV_BATCH at a time: the next batch's numbers are asked for before the
+// current batch is walked and put into LDS after it, so that the trip to memory runs beside the walk.
+// A request's rows in one walk, or in segments side by side (see lru_scan_kernel): carry [S, n_segs, H, d, d] holds what
+// a segment adds from zero and then the state that comes into it, cdec [S, n_segs, H, d] the product of its decays.
 struct WkvArgs {
     const elem_t* r;     // [T, H * d]
     const elem_t* k;
@@ -239,64 +299,139 @@ struct WkvArgs {
     const int* seq_slot;
     elem_t* out;         // [T, H * d]
     int H, d;
+    int seg_len, n_segs;
+    float* carry;
+    float* cdec;
 };
 
-template <int DP>
+constexpr int WKV_BATCH = 8;
+
+template <int DP, int MODE>
 __global__ __launch_bounds__(DP <= 64 ? 64 : 128) void wkv_kernel(WkvArgs a) {
-    constexpr int NT = DP <= 64 ? 64 : 128;
-    __shared__ float rs[2][DP], ks[2][DP], ws[2][DP];
-    __shared__ float scratch[NT / 64];
-    const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x, d = a.d, row = a.H * d;
-    const int q0 = a.seq_q_start[s], n = a.seq_q_len[s];
-    if (n <= 0) return;
+    constexpr int NT = DP <= 64 ? 64 : 128, NW = NT / 64, TB = WKV_BATCH;
+    __shared__ __align__(16) float rs[TB][DP], ks[TB][DP], ws[TB][DP];
+    __shared__ float vs[TB][NT], gs[TB][NT], bonus[TB][NW];
+    __shared__ float scratch[NW];
+    const int s = blockIdx.x, h = blockIdx.y, seg = blockIdx.z, j = threadIdx.x, d = a.d, row = a.H * d;
+    const int off = MODE == WALK_WHOLE ? 0 : seg * a.seg_len;
+    const int left = a.seq_q_len[s] - off;
+    if (left <= 0) return;
+    const int n = MODE == WALK_WHOLE ? left : min(left, a.seg_len);
+    const bool last = MODE == WALK_WHOLE || left <= a.seg_len;
+    if (MODE == WALK_LOCAL && last) return;  // nobody needs what the last segment passes on
+    const int q0 = a.seq_q_start[s] + off;
     const bool live = j < d;
     float* st = a.state + (((size_t)a.seq_slot[s] * a.H + h) * d) * d;
+    float* pass = MODE == WALK_WHOLE ? nullptr : a.carry + ((((size_t)s * a.n_segs + seg) * a.H + h) * d) * d;
     float S[DP];
+    {
+        const float* from = MODE == WALK_FINAL ? pass : st;
 #pragma unroll
-    for (int i = 0; i < DP; ++i) S[i] = (live && i < d) ? st[(size_t)i * d + j] : 0.f;
+        for (int i = 0; i < DP; ++i) S[i] = (MODE != WALK_LOCAL && live && i < d) ? from[(size_t)i * d + j] : 0.f;
+    }
     const int col = h * d + (live ? j : 0);
     const float w0 = a.w0[col], uj = a.u[col], nw = a.norm[col];
-    auto stage = [&](int b, int t) {  // this thread's key channel of token t
-        if (j < DP) {
-            const size_t at = (size_t)t * row + col;
-            rs[b][j] = live ? to_f32(a.r[at]) : 0.f;
-            ks[b][j] = live ? to_f32(a.k[at]) : 0.f;
-            ws[b][j] = live ? expf(-expf(a.z[at] + w0)) : 0.f;
+    float pr[TB], pk[TB], pz[TB], pv[TB], pg[TB];
+    auto fetch = [&](int j0) {  // this thread's channel of tokens j0 .. j0 + TB - 1 (the last one again beyond the end)
+#pragma unroll
+        for (int b = 0; b < TB; ++b) {
+            const size_t at = (size_t)(q0 + min(j0 + b, n - 1)) * row + col;
+            pk[b] = to_f32(a.k[at]);
+            pz[b] = a.z[at];
+            pv[b] = to_f32(a.v[at]);
+            if (MODE != WALK_LOCAL) {
+                pr[b] = to_f32(a.r[at]);
+                pg[b] = to_f32(a.gate[at]);
+            }
         }
     };
-    // the bonus belongs to the key channel: u[i] k[i]; kept beside k in LDS as r[i] u[i] k[i] would need r first
-    __shared__ float us[DP];
-    if (j < DP) us[j] = live ? uj : 0.f;
-    stage(0, q0);
-    __syncthreads();
-    for (int jt = 0; jt < n; ++jt) {
-        const int b = jt & 1, t = q0 + jt;
-        if (jt + 1 < n) stage(b ^ 1, t + 1);
-        const float vj = live ? to_f32(a.v[(size_t)t * row + col]) : 0.f;
-        float o = 0.f;
+    float pw = 1.f;  // the product of this key channel's decays over the segment
+    fetch(0);
+    for (int j0 = 0; j0 < n; j0 += TB) {
+        const int nb = min(TB, n - j0);
+        __syncthreads();  // the batch before has been walked by everyone
 #pragma unroll
-        for (int i = 0; i < DP; ++i) {
-            const float kv = ks[b][i] * vj;
-            o += rs[b][i] * (S[i] + us[i] * kv);
-            S[i] = ws[b][i] * S[i] + kv;
+        for (int b = 0; b < TB; ++b) {
+            const float w = live ? expf(-expf(pz[b] + w0)) : 0.f;
+            if (j < DP) {
+                ks[b][j] = live ? pk[b] : 0.f;
+                ws[b][j] = w;
+            }
+            vs[b][j] = live ? pv[b] : 0.f;
+            if (MODE == WALK_LOCAL) {
+                if (b < nb) pw *= w;
+            } else {
+                if (j < DP) rs[b][j] = live ? pr[b] : 0.f;
+                gs[b][j] = pg[b];
+                const float p = wave_sum(live ? pr[b] * uj * pk[b] : 0.f);
+                if ((j & 63) == 0) bonus[b][j >> 6] = p;
+            }
         }
-        float ss = live ? o * o : 0.f;
-        if constexpr (NT == 64) {
-            ss = wave_sum(ss);
-            __syncthreads();  // the next token's stage is written; this token's has been read by everyone
-        } else {
-            ss = block_sum<NT>(ss, scratch);  // its barriers do the same
-        }
-        if (live) {
-            const float g = to_f32(a.gate[(size_t)t * row + col]);
-            const float y = o / sqrtf(ss / (float)d + a.eps) * nw * (g / (1.0f + expf(-g)));
-            a.out[(size_t)t * row + col] = from_f32<elem_t>(y);
+        __syncthreads();
+        if (j0 + TB < n) fetch(j0 + TB);
+        for (int b = 0; b < nb; ++b) {
+            const float vj = vs[b][j];
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < DP; i += 4) {
+                const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][i]);
+                const float4 w4 = *reinterpret_cast<const float4*>(&ws[b][i]);
+                if (MODE != WALK_LOCAL) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(&rs[b][i]);
+                    o = fmaf(r4.x, S[i], o);
+                    o = fmaf(r4.y, S[i + 1], o);
+                    o = fmaf(r4.z, S[i + 2], o);
+                    o = fmaf(r4.w, S[i + 3], o);
+                }
+                S[i] = fmaf(w4.x, S[i], k4.x * vj);
+                S[i + 1] = fmaf(w4.y, S[i + 1], k4.y * vj);
+                S[i + 2] = fmaf(w4.z, S[i + 2], k4.z * vj);
+                S[i + 3] = fmaf(w4.w, S[i + 3], k4.w * vj);
+            }
+            if (MODE != WALK_LOCAL) {
+                float bn = bonus[b][0];
+                if constexpr (NW == 2) bn += bonus[b][1];
+                o = fmaf(bn, vj, o);
+                float ss = live ? o * o : 0.f;
+                if constexpr (NW == 1) ss = wave_sum(ss);
+                else ss = block_sum<NT>(ss, scratch);
+                if (live) {
+                    const float g = gs[b][j];
+                    const float y = o / sqrtf(ss / (float)d + a.eps) * nw * (g / (1.0f + expf(-g)));
+                    a.out[(size_t)(q0 + j0 + b) * row + col] = from_f32<elem_t>(y);
+                }
+            }
         }
     }
-    if (live) {
+    if (!live) return;
+    if (MODE == WALK_LOCAL) {
+#pragma unroll
+        for (int i = 0; i < DP; ++i)
+            if (i < d) pass[(size_t)i * d + j] = S[i];
+        a.cdec[(((size_t)s * a.n_segs + seg) * a.H + h) * d + j] = pw;
+    } else if (last) {
 #pragma unroll
         for (int i = 0; i < DP; ++i)
             if (i < d) st[(size_t)i * d + j] = S[i];
+    }
+}
+
+// Between the two passes: S_in(seg + 1) = diag(product of seg's decays) S_in(seg) + what seg adds, from the slot's state.
+__global__ __launch_bounds__(256) void wkv_carry_kernel(const float* __restrict__ state, const int* __restrict__ seq_q_len,
+                                                        const int* __restrict__ seq_slot, float* __restrict__ carry,
+                                                        const float* __restrict__ cdec, int H, int d, int seg_len, int n_segs) {
+    const int s = blockIdx.x, h = blockIdx.y, idx = blockIdx.z * 256 + threadIdx.x;
+    if (idx >= d * d) return;
+    const int i = idx / d;
+    const int nseg = (seq_q_len[s] + seg_len - 1) / seg_len;
+    float Sin = state[((size_t)seq_slot[s] * H + h) * d * d + idx];
+    for (int seg = 0; seg < nseg; ++seg) {
+        const size_t at = ((size_t)s * n_segs + seg) * H + h;
+        float* p = carry + at * d * d + idx;
+        const bool more = seg + 1 < nseg;
+        const float dec = more ? cdec[at * d + i] : 0.f, add = more ? *p : 0.f;
+        *p = Sin;
+        Sin = dec * Sin + add;
     }
 }
 
@@ -333,17 +468,32 @@ extern "C" int ms_lru_gates(const float* u, const void* wa_t, const void* wi_t, 
     const size_t lds = (size_t)GATE_ROWS * bw * sizeof(float);
     MS_REQUIRE(lds <= 64 * 1024, "lru_gates: blocks of %d channels exceed the rows' place in LDS", bw);
     GateArgs g{u, (const elem_t*)wa_t, (const elem_t*)wi_t, ba, bi, lam, c, a_out, drive_out, T, C, bw};
-    hipLaunchKernelGGL(lru_gates_kernel, dim3(ceil_div(T, GATE_ROWS), blocks), dim3(256), lds, stream, g);
+    hipLaunchKernelGGL(lru_gates_kernel, dim3(ceil_div(T, GATE_ROWS), blocks, ceil_div(bw, GATE_OUTS)), dim3(256), lds, stream, g);
     return check_launch("lru_gates");
 }
 
+// seg_len > 0: requests' rows in segments of seg_len that are walked side by side; n_segs covers the longest request of the
+// step, carry holds [S, n_segs, 2, C] floats.
 extern "C" int ms_lru_scan(const float* a, const float* drive, const void* y, int ldy, int ycol, const float* by, float* state,
-                           const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, void* out, int C,
-                           hipStream_t stream) {
+                           const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, void* out, int C, int seg_len,
+                           int n_segs, float* carry, hipStream_t stream) {
     MS_REQUIRE(S > 0 && C > 0 && ycol >= 0 && ycol + C <= ldy, "lru_scan: %d requests, %d channels at column %d of %d", S, C, ycol, ldy);
-    hipLaunchKernelGGL(lru_scan_kernel, dim3(S, ceil_div(C, 64)), dim3(64), 0, stream, a, drive, (const elem_t*)y, ldy, ycol, by,
-                       state, seq_q_start, seq_q_len, seq_slot, (elem_t*)out, C);
-    return check_launch("lru_scan");
+    MS_REQUIRE(seg_len == 0 || (seg_len > 0 && n_segs > 0 && carry), "lru_scan: segments of %d need their workspace", seg_len);
+#define MS_LRU(MODE, Z)                                                                                                          \
+    hipLaunchKernelGGL(lru_scan_kernel<MODE>, dim3(S, ceil_div(C, 64), Z), dim3(64), 0, stream, a, drive, (const elem_t*)y, ldy, \
+                       ycol, by, state, seq_q_start, seq_q_len, seq_slot, (elem_t*)out, C, seg_len, n_segs, carry)
+    if (seg_len == 0) {
+        MS_LRU(WALK_WHOLE, 1);
+        return check_launch("lru_scan");
+    }
+    MS_LRU(WALK_LOCAL, n_segs);
+    if (int rc = check_launch("lru_scan, segments from zero")) return rc;
+    hipLaunchKernelGGL(lru_carry_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, (const float*)state, seq_q_len, seq_slot,
+                       carry, C, seg_len, n_segs);
+    if (int rc = check_launch("lru_scan, states between segments")) return rc;
+    MS_LRU(WALK_FINAL, n_segs);
+#undef MS_LRU
+    return check_launch("lru_scan, segments");
 }
 
 extern "C" int ms_shift_mix(const float* x, float* prev, const float* mu, int M, const int* seq_q_start, const int* seq_q_len,
@@ -363,23 +513,38 @@ extern "C" int ms_tanh_rows(const float* in, void* out, long n, hipStream_t stre
     return check_launch("tanh_rows");
 }
 
+// seg_len > 0: as for ms_lru_scan; carry holds [S, n_segs, H, d, d] floats and cdec [S, n_segs, H, d].
 extern "C" int ms_wkv(const void* r, const void* k, const void* v, const void* gate, const float* z, const float* w0, const float* u,
                       const float* norm, float eps, float* state, const int* seq_q_start, const int* seq_q_len, const int* seq_slot,
-                      int S, void* out, int H, int d, hipStream_t stream) {
+                      int S, void* out, int H, int d, int seg_len, int n_segs, float* carry, float* cdec, hipStream_t stream) {
     MS_REQUIRE(S > 0 && H > 0 && d > 0 && d <= 128, "wkv: %d requests, %d heads of %d (at most 128)", S, H, d);
+    MS_REQUIRE(seg_len == 0 || (seg_len > 0 && n_segs > 0 && carry && cdec), "wkv: segments of %d need their workspace", seg_len);
     WkvArgs a{(const elem_t*)r, (const elem_t*)k, (const elem_t*)v, (const elem_t*)gate, z, w0, u, norm, eps, state,
-              seq_q_start, seq_q_len, seq_slot, (elem_t*)out, H, d};
-    const dim3 grid(S, H);
+              seq_q_start, seq_q_len, seq_slot, (elem_t*)out, H, d, seg_len, n_segs, carry, cdec};
     const int dp = ceil_div(d, 16) * 16;
-    switch (dp) {
-        case 16: hipLaunchKernelGGL(wkv_kernel<16>, grid, dim3(64), 0, stream, a); break;
-        case 32: hipLaunchKernelGGL(wkv_kernel<32>, grid, dim3(64), 0, stream, a); break;
-        case 48: hipLaunchKernelGGL(wkv_kernel<48>, grid, dim3(64), 0, stream, a); break;
-        case 64: hipLaunchKernelGGL(wkv_kernel<64>, grid, dim3(64), 0, stream, a); break;
-        case 80: hipLaunchKernelGGL(wkv_kernel<80>, grid, dim3(128), 0, stream, a); break;
-        case 96: hipLaunchKernelGGL(wkv_kernel<96>, grid, dim3(128), 0, stream, a); break;
-        case 112: hipLaunchKernelGGL(wkv_kernel<112>, grid, dim3(128), 0, stream, a); break;
-        default: hipLaunchKernelGGL(wkv_kernel<128>, grid, dim3(128), 0, stream, a); break;
+    auto walk = [&](auto mode, int Z) {
+        constexpr int MODE = decltype(mode)::value;
+        const dim3 grid(S, H, Z);
+        switch (dp) {
+            case 16: hipLaunchKernelGGL((wkv_kernel<16, MODE>), grid, dim3(64), 0, stream, a); break;
+            case 32: hipLaunchKernelGGL((wkv_kernel<32, MODE>), grid, dim3(64), 0, stream, a); break;
+            case 48: hipLaunchKernelGGL((wkv_kernel<48, MODE>), grid, dim3(64), 0, stream, a); break;
+            case 64: hipLaunchKernelGGL((wkv_kernel<64, MODE>), grid, dim3(64), 0, stream, a); break;
+            case 80: hipLaunchKernelGGL((wkv_kernel<80, MODE>), grid, dim3(128), 0, stream, a); break;
+            case 96: hipLaunchKernelGGL((wkv_kernel<96, MODE>), grid, dim3(128), 0, stream, a); break;
+            case 112: hipLaunchKernelGGL((wkv_kernel<112, MODE>), grid, dim3(128), 0, stream, a); break;
+            default: hipLaunchKernelGGL((wkv_kernel<128, MODE>), grid, dim3(128), 0, stream, a); break;
+        }
+    };
+    if (seg_len == 0) {
+        walk(std::integral_constant<int, WALK_WHOLE>{}, 1);
+        return check_launch("wkv");
     }
-    return check_launch("wkv");
+    walk(std::integral_constant<int, WALK_LOCAL>{}, n_segs);
+    if (int rc = check_launch("wkv, segments from zero")) return rc;
+    hipLaunchKernelGGL(wkv_carry_kernel, dim3(S, H, ceil_div(d * d, 256)), dim3(256), 0, stream, (const float*)state, seq_q_len,
+                       seq_slot, carry, (const float*)cdec, H, d, seg_len, n_segs);
+    if (int rc = check_launch("wkv, states between segments")) return rc;
+    walk(std::integral_constant<int, WALK_FINAL>{}, n_segs);
+    return check_launch("wkv, segments");
 }

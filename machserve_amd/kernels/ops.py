@@ -1127,9 +1127,28 @@ class HipOps:
         self._want(state, torch.float32, "lru state", state.shape[0], C)
         S = self._seq_operands("lru_scan", seq_q_start, seq_q_len, seq_slot)
         out = torch.empty((T, C), dtype=self.dtype, device=a.device)
+        seg, n_segs = self._walk_segments(T, S, self.LRU_SEGMENT, 2 * C)
+        carry = torch.empty((S, n_segs, 2, C), dtype=torch.float32, device=a.device) if seg else None
         self._check(lib, lib.ms_lru_scan(_ptr(a), _ptr(drive), _ptr(y), _c_int(y.shape[1]), _c_int(ycol), _ptr(y_bias), _ptr(state),
-                                         _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(C), self._stream()))
+                                         _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(C),
+                                         _c_int(seg), _c_int(n_segs), _ptr(carry), self._stream()))
         return out
+
+    LRU_SEGMENT = 64  # rows of a segment of the gated recurrence
+    WKV_SEGMENT = 32  # and of time mixing, whose walk does more a row
+
+    def _walk_segments(self, T: int, S: int, seg: int, floats_per_segment: int) -> tuple:
+        """``(segment length, segments a request)`` for a recurrence over a step of ``T`` rows in ``S`` requests, or ``(0, 0)``:
+        long portions are cut into segments that are walked side by side (each from zero, then each from the state that
+        comes into it), since one walk over a long prompt keeps a small part of the chip busy.  The cut follows from
+        the step's rows and requests alone."""
+        if T < self.SCAN_CHUNK_MIN_ROWS or T // S < self.SCAN_CHUNK_MIN_ROWS // 2:
+            return 0, 0
+        n_segs = -(-T // seg)
+        while S * n_segs * floats_per_segment * 4 > (256 << 20) and n_segs > 1:
+            seg *= 2
+            n_segs = -(-T // seg)
+        return (seg, n_segs) if n_segs > 1 else (0, 0)
 
     def shift_mix(self, x: torch.Tensor, prev: torch.Tensor, mu: torch.Tensor, seq_q_start: torch.Tensor, seq_q_len: torch.Tensor,
                   seq_slot: torch.Tensor) -> torch.Tensor:
@@ -1173,9 +1192,12 @@ class HipOps:
         self._want(state, torch.float32, "wkv state", state.shape[0], heads, dim, dim)
         S = self._seq_operands("wkv", seq_q_start, seq_q_len, seq_slot)
         out = torch.empty((T, n), dtype=self.dtype, device=r.device)
+        seg, n_segs = self._walk_segments(T, S, self.WKV_SEGMENT, heads * dim * dim)
+        carry = torch.empty((S, n_segs, heads, dim, dim), dtype=torch.float32, device=r.device) if seg else None
+        cdec = torch.empty((S, n_segs, heads, dim), dtype=torch.float32, device=r.device) if seg else None
         self._check(lib, lib.ms_wkv(_ptr(r), _ptr(k), _ptr(v), _ptr(gate), _ptr(z), _ptr(w0), _ptr(u), _ptr(norm_w), _c_float(eps), _ptr(state),
                                     _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(heads), _c_int(dim),
-                                    self._stream()))
+                                    _c_int(seg), _c_int(n_segs), _ptr(carry), _ptr(cdec), self._stream()))
         return out
 
     # ------------------------------------------------------------------ routed experts

@@ -104,10 +104,37 @@ def test_convolution_over_sums_in_one_step_and_in_many(C, taps, biases):
 @pytest.mark.parametrize("C,blocks", [(48, 3), (40, 5), (256, 1), (320, 4), (24, 24)])
 def test_gated_recurrence_in_one_step_and_in_many(dtype, C, blocks):
     """Gates and recurrence against the plain block with an identity convolution and projections."""
+    _gated_recurrence_case(dtype, C, blocks, [11, 1, 140], CUTS)
+
+
+def _short_segments(monkeypatch, ops, rows, lru, wkv):
+    """Steps of ``rows`` rows and more are walked in segments of ``lru`` and ``wkv`` rows."""
+    monkeypatch.setattr(type(ops), "SCAN_CHUNK_MIN_ROWS", rows)
+    monkeypatch.setattr(type(ops), "LRU_SEGMENT", lru)
+    monkeypatch.setattr(type(ops), "WKV_SEGMENT", wkv)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,blocks,seg", [(48, 3, 8), (320, 4, 5), (130, 1, 16)])
+def test_gated_recurrence_walked_in_segments(monkeypatch, dtype, C, blocks, seg):
+    """Requests of unequal lengths whose rows are walked in short segments side by side: a request of one segment, one that
+    ends on a segment's edge, one that ends just behind an edge; first whole, then the rest in portions that start
+    from a state."""
+    _short_segments(monkeypatch, ops_of(dtype), 2 * seg, seg, seg)
+    lens = [4 * seg, 3, 9 * seg + 1]
+    _gated_recurrence_case(dtype, C, blocks, lens, ([1000, 1000, 1000], [3 * seg - 1, 2, 4 * seg + 2], [2 * seg, 1, 2 * seg]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_recurrence_of_a_long_prompt(dtype):
+    """A prompt long enough for segments of the usual length, whole and in two portions, beside a short request."""
+    _gated_recurrence_case(dtype, 192, 3, [3, 1, 777], ([1000, 1000, 1000], [2, 1, 450]))
+
+
+def _gated_recurrence_case(dtype, C, blocks, lens, cuts_list):
     ops = ops_of(dtype)
     torch.manual_seed(C + blocks)
     bw = C // blocks
-    lens = [11, 1, 140]
     T = sum(lens)
     u = torch.randn(T, C)
     y = (torch.randn(T, C + 8)).to(dtype)
@@ -115,12 +142,13 @@ def test_gated_recurrence_in_one_step_and_in_many(dtype, C, blocks):
          "ri.b": torch.randn(blocks, bw), "lam": torch.randn(C) - 2.0, "y.b": torch.randn(C)}
     tp = {k: v.double() for k, v in t.items()}
     want = []
-    for s, n in zip([0, 11, 12], lens):
+    for s, n in zip([0, lens[0], lens[0] + lens[1]], lens):
         h = u[s:s + n].double()
         want.append(_plain_recurrence(h, y[s:s + n, 8:].double(), tp, C, blocks))
     want = torch.cat(want)
-    for cuts in CUTS:
-        state = torch.zeros(5, C, device=DEV)
+    for cuts in cuts_list:
+        state = torch.randn(5, C, device=DEV)  # a slot not yet used holds anything
+        state[1:4] = 0.0
         got = torch.zeros(T, C)
         for rows, q0, ql, slots, _ in _steps(lens, cuts):
             a, drive = ops.lru_gates(dev(u[rows]), dev(t["ra"].transpose(1, 2)), dev(t["ri"].transpose(1, 2)), dev(t["ra.b"].reshape(-1)),
@@ -159,10 +187,29 @@ def test_the_recurrences_gates_agree_with_the_plain_block():
 @pytest.mark.parametrize("H,d,width,rank", [(3, 16, 64, 8), (5, 8, 48, 12), (2, 64, 128, 32), (4, 48, 96, 16), (1, 128, 64, 8), (2, 80, 32, 8)])
 def test_time_mixing_in_one_step_and_in_many(dtype, H, d, width, rank):
     """Mixes, products, decay and the walk over the tokens, as the mixer strings them together, against the plain mixer."""
+    _time_mixing_case(dtype, H, d, width, rank, [11, 1, 90], CUTS)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,d,width,rank,seg", [(3, 16, 64, 8, 8), (2, 64, 128, 32, 5), (1, 128, 64, 8, 9), (2, 80, 32, 8, 16), (5, 8, 48, 12, 3)])
+def test_time_mixing_walked_in_segments(monkeypatch, dtype, H, d, width, rank, seg):
+    """As for the gated recurrence: short segments side by side, lengths on, behind and below a segment's edge, portions that
+    start from a state."""
+    _short_segments(monkeypatch, ops_of(dtype), 2 * seg, seg, seg)
+    lens = [4 * seg, 3, 9 * seg + 1]
+    _time_mixing_case(dtype, H, d, width, rank, lens, ([1000, 1000, 1000], [3 * seg - 1, 2, 4 * seg + 2], [2 * seg, 1, 2 * seg]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_time_mixing_of_a_long_prompt(dtype):
+    """A prompt long enough for segments of the usual length, whole and in two portions, beside a short request."""
+    _time_mixing_case(dtype, 3, 64, 96, 16, [3, 1, 600], ([1000, 1000, 1000], [2, 1, 333]))
+
+
+def _time_mixing_case(dtype, H, d, width, rank, lens, cuts_list):
     ops = ops_of(dtype)
     torch.manual_seed(H * d)
     n = H * d
-    lens = [11, 1, 90]
     T = sum(lens)
     x = torch.randn(T, width)
     t = {f"mu.{m}": torch.rand(width) for m in "rkvgw"}
@@ -171,13 +218,14 @@ def test_time_mixing_in_one_step_and_in_many(dtype, H, d, width, rank):
               "w0": torch.randn(n) * 0.5 - 2.0, "u": torch.randn(H, d) * 0.5, "norm": torch.rand(n) + 0.5, "o": torch.eye(n)})
     tp = {k: v.double() for k, v in t.items()}
     m = {"heads": H, "dim": d}
-    want = torch.cat([P.wkv(x[s:s + k].double(), tp, m, 1e-5) for s, k in zip([0, 11, 12], lens)])
+    want = torch.cat([P.wkv(x[s:s + k].double(), tp, m, 1e-5) for s, k in zip([0, lens[0], lens[0] + lens[1]], lens)])
     mu = torch.stack([t[f"mu.{s}"] for s in "rkvgw"])
     W = {k: dev(t[k], dtype) for k in ("r", "k", "v", "g", "w1", "w2")}
     fill = -rank % 8   # the products sum over multiples of 8: the mixer fills the bottleneck up with zeros, and so does this
     W["w1"], W["w2"] = torch.nn.functional.pad(W["w1"], (0, 0, 0, fill)).contiguous(), torch.nn.functional.pad(W["w2"], (0, fill)).contiguous()
-    for cuts in CUTS:
-        prev, state = torch.zeros(5, width, device=DEV), torch.zeros(5, H, d, d, device=DEV)
+    for cuts in cuts_list:
+        prev, state = torch.zeros(5, width, device=DEV), torch.randn(5, H, d, d, device=DEV)  # a slot not yet used holds anything
+        state[1:4] = 0.0
         got = torch.zeros(T, n)
         for rows, q0, ql, slots, _ in _steps(lens, cuts):
             seq = (i32(q0), i32(ql), i32(slots))
