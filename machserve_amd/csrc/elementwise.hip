@@ -275,8 +275,8 @@ __global__ __launch_bounds__(256) void pair_norm_add_kernel(float* __restrict__ 
 // product with biases, left as 32-bit sums
 __global__ __launch_bounds__(256) void gate_mul_kernel(const float* __restrict__ in, elem_t* __restrict__ out, int n, int act) {
     const size_t t = blockIdx.x;
-    for (int c = threadIdx.x; c < n; c += 256)
-        out[t * n + c] = from_f32<elem_t>(gate_activation(in[t * 2 * n + c], act) * in[t * 2 * n + n + c]);
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < n) out[t * n + c] = from_f32<elem_t>(gate_activation(in[t * 2 * n + c], act) * in[t * 2 * n + n + c]);
 }
 
 // out[t, :] = the stream's row in the element type: the input of a branch that reads the stream as it is.
@@ -614,7 +614,7 @@ extern "C" int ms_pair_norm_add(float* x, const float* pa, int na, const float* 
 extern "C" int ms_gate_mul(const float* in, void* out, int T, int n, int act, hipStream_t stream) {
     MS_REQUIRE(T > 0 && n > 0 && in && out, "gate_mul: empty problem T=%d n=%d", T, n);
     MS_REQUIRE(act >= 0 && act < ACT_COUNT, "gate_mul: activation %d", act);
-    hipLaunchKernelGGL(gate_mul_kernel, dim3(T), dim3(256), 0, stream, in, (elem_t*)out, n, act);
+    hipLaunchKernelGGL(gate_mul_kernel, dim3(T, ceil_div(n, 256)), dim3(256), 0, stream, in, (elem_t*)out, n, act);
     return check_launch("gate_mul");
 }
 

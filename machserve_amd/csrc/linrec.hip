@@ -68,10 +68,13 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs a) {
     const int keep = a.taps - 1;
     const float* st = a.state + (size_t)a.seq_slot[s] * keep * a.C;
     float acc = a.bias_out ? a.bias_out[c] : 0.f;
+    // both places are read for every tap, on one straight path (the loads go out together), and one is kept
+#pragma unroll 4
     for (int k = 0; k < a.taps; ++k) {
         const int back = keep - k, idx = j - back;
-        const float v = idx >= 0 ? conv_input(a, t - back, c) : st[(size_t)(keep + idx) * a.C + c];
-        acc += a.w[(size_t)c * a.taps + k] * v;
+        const float fresh = conv_input(a, t - min(back, j), c);
+        const float old = keep ? st[(size_t)min(max(keep + idx, 0), keep - 1) * a.C + c] : 0.f;
+        acc += a.w[(size_t)c * a.taps + k] * (idx >= 0 ? fresh : old);
     }
     a.out[(size_t)t * a.ld_out + a.out0 + c] = acc;
 }
@@ -110,36 +113,53 @@ struct GateArgs {
     int T, C, bw;
 };
 
+constexpr int GATE_K = 32;  // inputs whose weights a thread asks for at once
+
 __global__ __launch_bounds__(256) void lru_gates_kernel(GateArgs g) {
-    extern __shared__ float us[];  // [GATE_ROWS][bw]
+    extern __shared__ __align__(16) float us[];  // [GATE_ROWS][ldu], a row's end filled with zeros
     __shared__ float part[2][GATE_SLICES][GATE_ROWS][GATE_OUTS];
     const int t0 = blockIdx.x * GATE_ROWS, b = blockIdx.y, bw = g.bw;
+    const int ldu = (bw + 3) & ~3;
     const int nr = min(GATE_ROWS, g.T - t0);
-    for (int i = threadIdx.x; i < GATE_ROWS * bw; i += 256) {
-        const int r = i / bw, k = i - r * bw;
-        us[i] = r < nr ? g.u[(size_t)(t0 + r) * g.C + b * bw + k] : 0.f;
+    for (int i = threadIdx.x; i < GATE_ROWS * ldu; i += 256) {
+        const int r = i / ldu, k = i - r * ldu;
+        us[i] = (r < nr && k < bw) ? g.u[(size_t)(t0 + r) * g.C + b * bw + k] : 0.f;
     }
-    __syncthreads();
     const int lane = threadIdx.x & (GATE_OUTS - 1), slice = threadIdx.x / GATE_OUTS;
     const int o = blockIdx.z * GATE_OUTS + lane;
     const bool live = o < bw;
     const elem_t* wa = g.wa_t + (size_t)b * bw * bw + (live ? o : 0);
     const elem_t* wi = g.wi_t + (size_t)b * bw * bw + (live ? o : 0);
-    const int per = (bw + GATE_SLICES - 1) / GATE_SLICES;
-    const int k0 = slice * per, k1 = min(bw, k0 + per);
+    const int per = (((bw + GATE_SLICES - 1) / GATE_SLICES) + 3) & ~3;  // a slice's inputs, whole groups of four
+    const int k0 = slice * per, k1 = min(ldu, k0 + per);
     float ar[GATE_ROWS], ai[GATE_ROWS];
 #pragma unroll
     for (int r = 0; r < GATE_ROWS; ++r) ar[r] = ai[r] = 0.f;
-#pragma unroll 4
-    for (int k = k0; k < k1; ++k) {
-        const float fa = to_f32(wa[(size_t)k * bw]), fi = to_f32(wi[(size_t)k * bw]);
+    for (int kc = k0; kc < k1; kc += GATE_K) {
+        float fa[GATE_K], fi[GATE_K];
 #pragma unroll
-        for (int r = 0; r < GATE_ROWS; ++r) {
-            const float uv = us[r * bw + k];
-            ar[r] += fa * uv;
-            ai[r] += fi * uv;
+        for (int q = 0; q < GATE_K; ++q) {  // the weights of GATE_K inputs in one trip to memory
+            const int k = kc + q;
+            const bool in = k < k1 && k < bw;
+            const size_t at = (size_t)min(k, bw - 1) * bw;  // every load goes out, on one straight path
+            const float va = to_f32(wa[at]), vi = to_f32(wi[at]);
+            fa[q] = in ? va : 0.f;
+            fi[q] = in ? vi : 0.f;
+        }
+        if (kc == k0) __syncthreads();  // the rows are in LDS (the first weights were asked for meanwhile)
+#pragma unroll
+        for (int q = 0; q < GATE_K; q += 4) {
+            if (kc + q < k1) {
+#pragma unroll
+                for (int r = 0; r < GATE_ROWS; ++r) {
+                    const float4 u4 = *reinterpret_cast<const float4*>(&us[r * ldu + kc + q]);
+                    ar[r] += fa[q] * u4.x + fa[q + 1] * u4.y + fa[q + 2] * u4.z + fa[q + 3] * u4.w;
+                    ai[r] += fi[q] * u4.x + fi[q + 1] * u4.y + fi[q + 2] * u4.z + fi[q + 3] * u4.w;
+                }
+            }
         }
     }
+    if (k0 >= k1) __syncthreads();  // a slice without inputs has not met the others yet
 #pragma unroll
     for (int r = 0; r < GATE_ROWS; ++r) {
         part[0][slice][r][lane] = ar[r];
@@ -161,7 +181,7 @@ __global__ __launch_bounds__(256) void lru_gates_kernel(GateArgs g) {
         const float log_a = -g.c * rg * sp;
         const float av = expf(log_a);
         // 1 - a^2 = -expm1(2 log a): no cancellation where a is close to one
-        const float drive = sqrtf(-expm1f(2.0f * log_a)) * ig * us[r * bw + o];
+        const float drive = sqrtf(-expm1f(2.0f * log_a)) * ig * us[r * ldu + o];
         g.a_out[(size_t)(t0 + r) * g.C + c] = av;
         g.drive_out[(size_t)(t0 + r) * g.C + c] = drive;
     }
@@ -250,10 +270,10 @@ __global__ __launch_bounds__(256) void shift_mix_kernel(const float* __restrict_
     const int s = seq_of_row(t, seq_q_start, S);
     const float* before = t > seq_q_start[s] ? x + (size_t)(t - 1) * d : prev + (size_t)seq_slot[s] * d;
     const float* cur = x + (size_t)t * d;
-    for (int c = threadIdx.x; c < d; c += 256) {
-        const float v = cur[c], dlt = before[c] - v;
-        for (int m = 0; m < M; ++m) out[((size_t)m * T + t) * d + c] = from_f32<elem_t>(v + dlt * mu[(size_t)m * d + c]);
-    }
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= d) return;
+    const float v = cur[c], dlt = before[c] - v;
+    for (int m = 0; m < M; ++m) out[((size_t)m * T + t) * d + c] = from_f32<elem_t>(v + dlt * mu[(size_t)m * d + c]);
 }
 
 // prev[slot of request s] = its last row of the step
@@ -465,7 +485,7 @@ extern "C" int ms_lru_gates(const float* u, const void* wa_t, const void* wi_t, 
                             float c, float* a_out, float* drive_out, int T, int C, int blocks, hipStream_t stream) {
     MS_REQUIRE(T > 0 && C > 0 && blocks > 0 && C % blocks == 0, "lru_gates: %d channels in %d blocks, %d rows", C, blocks, T);
     const int bw = C / blocks;
-    const size_t lds = (size_t)GATE_ROWS * bw * sizeof(float);
+    const size_t lds = (size_t)GATE_ROWS * ((bw + 3) & ~3) * sizeof(float);
     MS_REQUIRE(lds <= 64 * 1024, "lru_gates: blocks of %d channels exceed the rows' place in LDS", bw);
     GateArgs g{u, (const elem_t*)wa_t, (const elem_t*)wi_t, ba, bi, lam, c, a_out, drive_out, T, C, bw};
     hipLaunchKernelGGL(lru_gates_kernel, dim3(ceil_div(T, GATE_ROWS), blocks, ceil_div(bw, GATE_OUTS)), dim3(256), lds, stream, g);
@@ -499,7 +519,7 @@ extern "C" int ms_lru_scan(const float* a, const float* drive, const void* y, in
 extern "C" int ms_shift_mix(const float* x, float* prev, const float* mu, int M, const int* seq_q_start, const int* seq_q_len,
                             const int* seq_slot, int S, void* out, int T, int d, hipStream_t stream) {
     MS_REQUIRE(T > 0 && d > 0 && S > 0 && M > 0, "shift_mix: empty problem T=%d d=%d S=%d M=%d", T, d, S, M);
-    hipLaunchKernelGGL(shift_mix_kernel, dim3(T), dim3(256), 0, stream, x, (const float*)prev, mu, M, seq_q_start, seq_slot, S,
+    hipLaunchKernelGGL(shift_mix_kernel, dim3(T, ceil_div(d, 256)), dim3(256), 0, stream, x, (const float*)prev, mu, M, seq_q_start, seq_slot, S,
                        (elem_t*)out, T, d);
     int rc = check_launch("shift_mix");
     if (rc) return rc;

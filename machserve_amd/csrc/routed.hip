@@ -24,6 +24,7 @@ __global__ __launch_bounds__(256) void route_kernel(const elem_t* __restrict__ x
     for (int e = wave; e < E; e += 4) {
         const float* we = w + (size_t)e * d;
         float acc = 0.f;
+#pragma unroll 8
         for (int c = lane; c < d; c += 64) acc += to_f32(row[c]) * we[c];
         acc = wave_sum(acc);
         if (lane == 0) z[e] = acc + (bias ? bias[e] : 0.f);
@@ -71,11 +72,13 @@ __device__ __forceinline__ float expert_activation(float z, int act) {
 }
 
 // a[t, c] = act(up[t, c]) * gates[t, c / ff] for c < E * ff, act(up[t, c]) beyond (experts that every row uses)
+constexpr int ACT_COLS = 2048;  // columns of a row that a block takes
 __global__ __launch_bounds__(256) void expert_act_kernel(const float* __restrict__ up, const float* __restrict__ gates,
                                                          elem_t* __restrict__ out, int n, int E, int ff, int act) {
-    const int t = blockIdx.x;
+    const int t = blockIdx.x, c0 = blockIdx.y * ACT_COLS, c1 = min(n, c0 + ACT_COLS);
     const float* g = gates + (size_t)t * E;
-    for (int c = threadIdx.x; c < n; c += 256) {
+#pragma unroll 4
+    for (int c = c0 + threadIdx.x; c < c1; c += 256) {
         const int e = c / ff;
         const float w = e < E ? g[e] : 1.0f;
         // an expert the row did not choose contributes an exact zero, whatever its product holds
@@ -100,6 +103,6 @@ extern "C" int ms_route(const void* x, const float* w, const float* bias, float*
 extern "C" int ms_expert_act(const float* up, const float* gates, void* out, int T, int n, int E, int ff, int act, hipStream_t stream) {
     MS_REQUIRE(T > 0 && n > 0 && E >= 0 && ff > 0 && (long)E * ff <= n, "expert_act: %d columns for %d experts of %d", n, E, ff);
     MS_REQUIRE(act >= 0 && act <= 2, "expert_act: activation %d", act);
-    hipLaunchKernelGGL(expert_act_kernel, dim3(T), dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
+    hipLaunchKernelGGL(expert_act_kernel, dim3(T, ceil_div(n, ACT_COLS)), dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
     return check_launch("expert_act");
 }
