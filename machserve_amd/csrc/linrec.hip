@@ -68,13 +68,21 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(ConvArgs a) {
     const int keep = a.taps - 1;
     const float* st = a.state + (size_t)a.seq_slot[s] * keep * a.C;
     float acc = a.bias_out ? a.bias_out[c] : 0.f;
-    // both places are read for every tap, on one straight path (the loads go out together), and one is kept
+    // a tap reads the step's rows or the state (which of the two is the same for the whole block); the address is chosen,
+    // not the load: every load goes out on one straight path
+    const float bias = a.bias_in ? a.bias_in[c] : 0.f;
 #pragma unroll 4
     for (int k = 0; k < a.taps; ++k) {
         const int back = keep - k, idx = j - back;
-        const float fresh = conv_input(a, t - min(back, j), c);
-        const float old = keep ? st[(size_t)min(max(keep + idx, 0), keep - 1) * a.C + c] : 0.f;
-        acc += a.w[(size_t)c * a.taps + k] * (idx >= 0 ? fresh : old);
+        const bool fresh = idx >= 0;
+        const float* src = fresh ? a.in + (size_t)(t - back) * a.ld + a.col0 + c : st + (size_t)(keep + idx) * a.C + c;
+        const size_t stride = fresh ? a.partial_stride : 0;
+        float v = fresh ? bias : 0.f;
+        for (int p = 0; p < a.n_partials; ++p) {
+            const float part = src[p * stride];
+            v += (fresh || p == 0) ? part : 0.f;
+        }
+        acc += a.w[(size_t)c * a.taps + k] * v;
     }
     a.out[(size_t)t * a.ld_out + a.out0 + c] = acc;
 }
@@ -331,7 +339,7 @@ __global__ __launch_bounds__(DP <= 64 ? 64 : 128) void wkv_kernel(WkvArgs a) {
     constexpr int NT = DP <= 64 ? 64 : 128, NW = NT / 64, TB = WKV_BATCH;
     __shared__ __align__(16) float rs[TB][DP], ks[TB][DP], ws[TB][DP];
     __shared__ float vs[TB][NT], gs[TB][NT], bonus[TB][NW];
-    __shared__ float scratch[NW];
+    __shared__ float os[TB][NT], halves[TB][2];
     const int s = blockIdx.x, h = blockIdx.y, seg = blockIdx.z, j = threadIdx.x, d = a.d, row = a.H * d;
     const int off = MODE == WALK_WHOLE ? 0 : seg * a.seg_len;
     const int left = a.seq_q_len[s] - off;
@@ -389,35 +397,57 @@ __global__ __launch_bounds__(DP <= 64 ? 64 : 128) void wkv_kernel(WkvArgs a) {
         }
         __syncthreads();
         if (j0 + TB < n) fetch(j0 + TB);
+        // the batch's outputs wait in LDS, each in its thread's own place: their norms are worked out together behind the walk
+#pragma unroll 1
         for (int b = 0; b < nb; ++b) {
-            const float vj = vs[b][j];
-            float o = 0.f;
+            {
+                const float vj = vs[b][j];
+                float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;  // four chains of sums side by side
 #pragma unroll
-            for (int i = 0; i < DP; i += 4) {
-                const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][i]);
-                const float4 w4 = *reinterpret_cast<const float4*>(&ws[b][i]);
-                if (MODE != WALK_LOCAL) {
-                    const float4 r4 = *reinterpret_cast<const float4*>(&rs[b][i]);
-                    o = fmaf(r4.x, S[i], o);
-                    o = fmaf(r4.y, S[i + 1], o);
-                    o = fmaf(r4.z, S[i + 2], o);
-                    o = fmaf(r4.w, S[i + 3], o);
+                for (int i = 0; i < DP; i += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(&ks[b][i]);
+                    const float4 w4 = *reinterpret_cast<const float4*>(&ws[b][i]);
+                    if (MODE != WALK_LOCAL) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(&rs[b][i]);
+                        o0 = fmaf(r4.x, S[i], o0);
+                        o1 = fmaf(r4.y, S[i + 1], o1);
+                        o2 = fmaf(r4.z, S[i + 2], o2);
+                        o3 = fmaf(r4.w, S[i + 3], o3);
+                    }
+                    S[i] = fmaf(w4.x, S[i], k4.x * vj);
+                    S[i + 1] = fmaf(w4.y, S[i + 1], k4.y * vj);
+                    S[i + 2] = fmaf(w4.z, S[i + 2], k4.z * vj);
+                    S[i + 3] = fmaf(w4.w, S[i + 3], k4.w * vj);
                 }
-                S[i] = fmaf(w4.x, S[i], k4.x * vj);
-                S[i + 1] = fmaf(w4.y, S[i + 1], k4.y * vj);
-                S[i + 2] = fmaf(w4.z, S[i + 2], k4.z * vj);
-                S[i + 3] = fmaf(w4.w, S[i + 3], k4.w * vj);
+                if (MODE != WALK_LOCAL) {
+                    float bn = bonus[b][0];
+                    if constexpr (NW == 2) bn += bonus[b][1];
+                    os[b][j] = fmaf(bn, vj, (o0 + o1) + (o2 + o3));
+                }
             }
-            if (MODE != WALK_LOCAL) {
-                float bn = bonus[b][0];
-                if constexpr (NW == 2) bn += bonus[b][1];
-                o = fmaf(bn, vj, o);
-                float ss = live ? o * o : 0.f;
-                if constexpr (NW == 1) ss = wave_sum(ss);
-                else ss = block_sum<NT>(ss, scratch);
-                if (live) {
+        }
+        if (MODE != WALK_LOCAL) {
+            float ob[TB], ss[TB];
+#pragma unroll
+            for (int b = 0; b < TB; ++b) {
+                ob[b] = (live && b < nb) ? os[b][j] : 0.f;
+                ss[b] = wave_sum(ob[b] * ob[b]);
+            }
+            if constexpr (NW == 2) {  // the head's other half
+                __syncthreads();
+                if ((j & 63) == 0) {
+#pragma unroll
+                    for (int b = 0; b < TB; ++b) halves[b][j >> 6] = ss[b];
+                }
+                __syncthreads();
+#pragma unroll
+                for (int b = 0; b < TB; ++b) ss[b] = halves[b][0] + halves[b][1];
+            }
+#pragma unroll
+            for (int b = 0; b < TB; ++b) {
+                if (live && b < nb) {
                     const float g = gs[b][j];
-                    const float y = o / sqrtf(ss / (float)d + a.eps) * nw * (g / (1.0f + expf(-g)));
+                    const float y = ob[b] / sqrtf(ss[b] / (float)d + a.eps) * nw * (g / (1.0f + expf(-g)));
                     a.out[(size_t)(q0 + j0 + b) * row + col] = from_f32<elem_t>(y);
                 }
             }

@@ -73,16 +73,27 @@ __device__ __forceinline__ float expert_activation(float z, int act) {
 
 // a[t, c] = act(up[t, c]) * gates[t, c / ff] for c < E * ff, act(up[t, c]) beyond (experts that every row uses)
 constexpr int ACT_COLS = 2048;  // columns of a row that a block takes
+template <int V>  // columns a thread takes at once: 4 where an expert's columns and the row are multiples of four
 __global__ __launch_bounds__(256) void expert_act_kernel(const float* __restrict__ up, const float* __restrict__ gates,
                                                          elem_t* __restrict__ out, int n, int E, int ff, int act) {
     const int t = blockIdx.x, c0 = blockIdx.y * ACT_COLS, c1 = min(n, c0 + ACT_COLS);
     const float* g = gates + (size_t)t * E;
-#pragma unroll 4
-    for (int c = c0 + threadIdx.x; c < c1; c += 256) {
+#pragma unroll 2
+    for (int c = c0 + threadIdx.x * V; c < c1; c += 256 * V) {
         const int e = c / ff;
         const float w = e < E ? g[e] : 1.0f;
         // an expert the row did not choose contributes an exact zero, whatever its product holds
-        out[(size_t)t * n + c] = from_f32<elem_t>(w != 0.f ? expert_activation(up[(size_t)t * n + c], act) * w : 0.f);
+        if constexpr (V == 4) {
+            float4 v = (float4){0.f, 0.f, 0.f, 0.f};
+            if (w != 0.f) v = *reinterpret_cast<const float4*>(up + (size_t)t * n + c);
+            elem_t* o = out + (size_t)t * n + c;
+            o[0] = from_f32<elem_t>(w != 0.f ? expert_activation(v.x, act) * w : 0.f);
+            o[1] = from_f32<elem_t>(w != 0.f ? expert_activation(v.y, act) * w : 0.f);
+            o[2] = from_f32<elem_t>(w != 0.f ? expert_activation(v.z, act) * w : 0.f);
+            o[3] = from_f32<elem_t>(w != 0.f ? expert_activation(v.w, act) * w : 0.f);
+        } else {
+            out[(size_t)t * n + c] = from_f32<elem_t>(w != 0.f ? expert_activation(up[(size_t)t * n + c], act) * w : 0.f);
+        }
     }
 }
 
@@ -103,6 +114,8 @@ extern "C" int ms_route(const void* x, const float* w, const float* bias, float*
 extern "C" int ms_expert_act(const float* up, const float* gates, void* out, int T, int n, int E, int ff, int act, hipStream_t stream) {
     MS_REQUIRE(T > 0 && n > 0 && E >= 0 && ff > 0 && (long)E * ff <= n, "expert_act: %d columns for %d experts of %d", n, E, ff);
     MS_REQUIRE(act >= 0 && act <= 2, "expert_act: activation %d", act);
-    hipLaunchKernelGGL(expert_act_kernel, dim3(T, ceil_div(n, ACT_COLS)), dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
+    const dim3 grid(T, ceil_div(n, ACT_COLS));
+    if (n % 4 == 0 && ff % 4 == 0) hipLaunchKernelGGL(expert_act_kernel<4>, grid, dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
+    else hipLaunchKernelGGL(expert_act_kernel<1>, grid, dim3(256), 0, stream, up, gates, (elem_t*)out, n, E, ff, act);
     return check_launch("expert_act");
 }
