@@ -481,6 +481,18 @@ def test_a_long_prompt_in_portions_behind_pages_of_64(tmp_path):
         assert U.relative_error(got, want) < F32, what
 
 
+def test_long_portions_beside_decoded_tokens(tmp_path):
+    """Steps whose rows are many enough for the recurrences' segments while some requests bring one row: two long
+    portions side by side, then a long portion beside two requests that decode."""
+    d = U.make_dir(tmp_path, "mixed", seed=21)
+    reqs = {"a": U.tokens_of(700, 97, 1), "b": U.tokens_of(420, 97, 2), "c": U.tokens_of(9, 97, 3)}
+    schedule = [[("a", 290), ("b", 300)], [("c", 7), ("b", 118)], [("b", 1), ("a", 405), ("c", 1)], [("b", 1), ("a", 5), ("c", 1)]]
+    lm = loaded(d, torch.float32, page_size=64, max_tokens=1344, max_requests=3)
+    got = U.run_schedule(lm, reqs, schedule)
+    for i, toks in reqs.items():
+        assert U.relative_error(got[i], plain_for(d, torch.float32, toks)) < F32, i
+
+
 def test_first_tokens_of_a_sequence(tmp_path):
     for name in sorted(U.CONFIGS):
         d = U.make_dir(tmp_path, name, seed=12)
