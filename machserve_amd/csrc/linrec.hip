@@ -8,8 +8,9 @@
 // seq_q_len); a request's state lives in slot seq_slot[s] of arrays [slots, ...] of 32-bit floats, is read at the start
 // of the request's rows and written back after its last.  Gates, decays and their logarithms, exponentials, the states
 // and every sum are 32-bit in every build; the element type stores what the next matrix product reads.  A row's result
-// depends on its own request alone, and on how its tokens were cut into steps not at all: every walk is token after
-// token in the same order.
+// depends on its own request alone.  Short steps walk a request's rows token after token; long portions are walked in
+// segments side by side whose incoming states a carry kernel chains, so that cuts of a prompt differ by that chain's
+// 32-bit rounding and by nothing else.
 #include "common.cuh"
 #include <type_traits>
 

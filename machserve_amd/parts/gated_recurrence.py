@@ -4,7 +4,8 @@ Per step: the gate branch ``y = W_y h`` in the element type and the recurrent br
 convolution per channel over the recurrent branch (its last ``taps - 1`` inputs are state; the projection's bias enters
 before it, the convolution's own after it); per block of channels the two gates from square maps of the convolved
 input, the decay ``a = exp(-c r softplus(lam))`` and the drive ``sqrt(1 - a^2) i u``; the recurrence ``S <- a S + drive``
-token after token from the request's slot, times ``gelu_tanh(y + b_y)``; the output projection.  Gates, decays, the
+token after token from the request's slot (long portions in segments side by side, see ``ops.lru_scan``), times
+``gelu_tanh(y + b_y)``; the output projection.  Gates, decays, the
 state and the convolution are 32-bit in every build.
 """
 from __future__ import annotations

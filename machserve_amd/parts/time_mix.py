@@ -4,7 +4,7 @@ Per step: each of r, k, v, the gate and the decay reads its own mix of a token's
 (``x + (x' - x) mu``, worked out from the 32-bit stream; the previous token's input is state); four products for r, k, v
 and the gate; the decay's bottleneck (product, tanh, product, left as 32-bit sums); one kernel that walks a request's
 tokens per head with the ``[dim, dim]`` state in registers (``o = (S + diag(u) k v^T)^T r``, ``S <- diag(w) S + k v^T`` with
-``w = exp(-exp(z + w0))``), divides a head's output by its root mean square, and applies the weight and the gate's SiLU;
+``w = exp(-exp(z + w0))``; long portions in segments side by side, see ``ops.wkv``), divides a head's output by its root mean square, and applies the weight and the gate's SiLU;
 the output projection.  The decay, the state and the unit norm are 32-bit in every build.
 """
 from __future__ import annotations
