@@ -492,6 +492,7 @@ using namespace ms;
 
 extern "C" int ms_linrec_max_taps() { return MAX_TAPS; }
 extern "C" int ms_wkv_max_dim() { return 128; }
+extern "C" int ms_lru_max_block() { return 64 * 1024 / (GATE_ROWS * (int)sizeof(float)); }  // a block's rows lie in LDS
 
 // One launch for the convolution and one for the state, in this order: the first reads the state that the second
 // replaces.  `out` may not alias `in`.

@@ -1061,7 +1061,7 @@ class HipOps:
     # ------------------------------------------------------------------ linear recurrences with gates that depend on the token
     def linrec_limits(self) -> dict:
         lib = self._extra_lib("linrec")
-        return {"taps": lib.ms_linrec_max_taps(), "wkv_dim": lib.ms_wkv_max_dim()}
+        return {"taps": lib.ms_linrec_max_taps(), "wkv_dim": lib.ms_wkv_max_dim(), "lru_block": lib.ms_lru_max_block()}
 
     def conv_sums(self, sums: torch.Tensor, col0: int, channels: int, bias_in: Optional[torch.Tensor], weight: torch.Tensor,
                   bias_out: Optional[torch.Tensor], state: Optional[torch.Tensor], seq_q_start: torch.Tensor, seq_q_len: torch.Tensor,

@@ -30,6 +30,8 @@ class GatedRecurrence(Mixer):
         if limits is not None and s.conv_taps > limits()["taps"]:
             raise ValueError(f"gated_recurrence: {s.conv_taps} taps; the convolution takes up to {limits()['taps']}")
         self.bw = s.width // s.blocks
+        if limits is not None and self.bw > limits().get("lru_block", self.bw):
+            raise ValueError(f"gated_recurrence: blocks of {self.bw} channels; the gates' kernel takes up to {limits()['lru_block']}")
         self.state = None
 
     def tensor_decls(self):

@@ -356,7 +356,7 @@ class EmulatedOps:
 
     # ------------------------------------------------------------------ linear recurrences with gates that depend on the token
     def linrec_limits(self):
-        return {"taps": 16, "wkv_dim": 128}
+        return {"taps": 16, "wkv_dim": 128, "lru_block": 1024}
 
     def conv_sums(self, sums, col0, channels, bias_in, weight, bias_out, state, seq_q_start, seq_q_len, seq_slot):
         row = (sums.sum(0) if sums.dim() == 3 else sums)[:, col0:col0 + channels]

@@ -493,6 +493,20 @@ def test_long_portions_beside_decoded_tokens(tmp_path):
         assert U.relative_error(got[i], plain_for(d, torch.float32, toks)) < F32, i
 
 
+def test_sizes_the_recurrences_do_not_take_are_refused_when_the_part_is_built():
+    """Blocks of the recurrence wider than the gates' kernel holds, and heads of time mixing beyond its registers, are
+    refused with the size when the part is built, not at the first step."""
+    from machserve_amd.config import GatedRecurrenceSpec, TimeMixSpec
+    from machserve_amd.parts import MIXERS, Runtime
+    rt = Runtime(torch.device(DEV), torch.bfloat16, ops_of(torch.bfloat16))
+    most = rt.ops.linrec_limits()["lru_block"]
+    MIXERS.build(GatedRecurrenceSpec("gated_recurrence", 64, 2 * most, 2, 4), rt)
+    with pytest.raises(ValueError, match=f"blocks of {2 * most}"):
+        MIXERS.build(GatedRecurrenceSpec("gated_recurrence", 64, 2 * most, 1, 4), rt)
+    with pytest.raises(ValueError, match="heads of 136"):
+        MIXERS.build(TimeMixSpec("time_mix", 64, 2, 136, 8, 1e-5), rt)
+
+
 def test_first_tokens_of_a_sequence(tmp_path):
     for name in sorted(U.CONFIGS):
         d = U.make_dir(tmp_path, name, seed=12)
