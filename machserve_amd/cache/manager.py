@@ -152,8 +152,8 @@ class CacheManager:
                 elif r is not None:
                     raise CacheError(f"layer {i}: unknown cache request {r!r}")
         for (i, j), src in self.shared.items():
-            if (src, 0) not in self.paged or self.layer_requests[src][0]:
-                raise CacheError(f"layer {i} reads the cache of layer {src}, which keeps no single paged cache")
+            if (src, 0) not in self.paged:  # a layer that asks for several things names its pages first
+                raise CacheError(f"layer {i} reads the cache of layer {src}, which keeps no paged cache (or does not ask for it first)")
         # the one-request view, as most layers have it
         self.layer_group = {i: g for (i, j), g in self.paged.items() if not self.layer_requests[i][0]}
         self.layer_source = {i: src for (i, j), src in self.shared.items() if not self.layer_requests[i][0]}

@@ -162,6 +162,56 @@ class LatentAttentionSpec:
     sink: bool = False
     kv_source: Optional[int] = None
     tensors: Mapping[str, str] = field(default_factory=dict)
+    # ``q_rank`` 0: no bottleneck, the heads' queries are one projection of the input ("q.weight")
+    # a row at position i sees the keys j with ``0 <= i - j < window`` (None: every j <= i)
+    window: Optional[int] = None
+    # a head's output is multiplied by the sigmoid of one number a head, a projection of the mixer's input ("g.weight")
+    head_gate: bool = False
+
+
+@dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Differential grouped-query attention: every head has two softmax maps over the same values, each with queries and
+    keys of its own (q is ``heads x 2 x head_dim``, k ``kv_heads x 2 x head_dim``, a head's two maps side by side), and its
+    result is ``a1 - lambda a2`` with ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff`` one number a layer, divided by its
+    root mean square over the head's ``v_head_dim`` values (``norm_eps``, no weight) and multiplied by ``1 - diff``; the
+    heads side by side are multiplied by ``sigmoid(W_g h)`` and projected.  With ``conv_taps`` > 0 a causal convolution
+    over time on every channel of q, k and v comes right behind the projections (no bias; the last ``conv_taps - 1``
+    inputs are a request's state); ``position``: the rotation of every map of q and k.  ``kv_source``: index of another
+    such layer whose keys and values this layer reads instead of having its own."""
+    kind: str
+    hidden: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    diff: float
+    position: Optional[RotarySpec] = None
+    conv_taps: int = 0
+    bias: bool = True
+    norm_eps: float = 1e-6
+    kv_source: Optional[int] = None
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class StateSpaceDualSpec:
+    """The second Mamba layer: ``heads`` heads of ``head_dim`` value channels with a state of ``states x head_dim`` each,
+    ``S <- exp(-exp(A_log) dt) S + dt B x^T``, ``y = S^T C + D x`` with one step size a head and token (``dt = softplus(. +
+    dt_bias)``) and B and C shared by the heads of a group.  The input projection is ``[z | x | B | C | dt]``; x, B and C
+    pass a causal convolution of ``conv_taps`` per channel with bias and SiLU; ``y silu(z)`` is RMS-normed in
+    ``norm_groups`` equal parts (``norm_eps``, a weight per channel) and projected."""
+    kind: str
+    hidden: int
+    heads: int
+    head_dim: int
+    states: int
+    groups: int
+    conv_taps: int
+    norm_groups: int = 1
+    norm_eps: float = 1e-6
+    tensors: Mapping[str, str] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)
@@ -278,6 +328,15 @@ class RoutedMlpSpec:
     shared: int = 0
     router_bias: bool = True
     tensors: Mapping[str, str] = field(default_factory=dict)
+    # an expert is ``W_down (act(W_gate h) * (W_up h))`` ("e<i>.gate" beside "e<i>.up")
+    gated: bool = False
+    # the router has this many outputs more, which stand for experts without tensors that return their input
+    identity: int = 0
+    # "softmax_chosen": the weights are the softmax over the chosen logits; "softmax_all": scores are the softmax over
+    # every router output, and the weights the chosen scores over their sum (+ 1e-20)
+    scoring: str = "softmax_chosen"
+    # with "softmax_all": a vector ("correction") added to the scores for the choice only
+    correction: bool = False
 
 
 @dataclass(frozen=True)
@@ -325,6 +384,29 @@ class PostNormLayerSpec:
     feed_forward: Optional[object]
     mixer_post_norm: object
     feed_forward_post_norm: Optional[object]
+
+
+@dataclass(frozen=True)
+class StreamMixSpec:
+    """How one branch reads and writes several residual streams: ``u = sum_s in[s] x_s`` is the branch's input, and all
+    streams at once become ``x_t = sum_s mix[s, t] x_s + out[t] y``."""
+    streams: int
+    tensors: Mapping[str, str] = field(default_factory=dict)
+    kind: str = "stream_mix"
+
+
+@dataclass(frozen=True)
+class MultiStreamLayerSpec:
+    """A pre-norm block over several residual streams: each branch reads a weighted sum of the streams through its norm
+    and is written back into all of them (``mixer_streams``, ``feed_forward_streams``); ``feed_forward`` None: the layer
+    has none."""
+    block: str
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_norm: object
+    feed_forward_norm: Optional[object]
+    mixer_streams: StreamMixSpec
+    feed_forward_streams: Optional[StreamMixSpec]
 
 
 @dataclass(frozen=True)
@@ -382,6 +464,8 @@ class ModelSpec:
     final_norm: object
     head: HeadSpec
     max_positions: int
+    # several residual streams, all equal to the embedding at the start and summed at the end (None: the one stream)
+    streams: Optional[int] = None
 
     def validate(self) -> None:
         n = len(self.layers)

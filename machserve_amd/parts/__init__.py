@@ -1,9 +1,9 @@
-from .base import (Block, FeedForward, GroupView, Mixer, Norm, PagedKVRequest, Part, PendingNorm, PositionEncoding, ResidualStream, Runtime,
+from .base import (Block, FeedForward, GroupView, Mixer, MultiStream, Norm, PagedKVRequest, Part, PendingNorm, PositionEncoding, ResidualStream, Runtime,
                    SharedKVRequest, StateRequest, StepContext, TensorDecl)
 from .registry import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, register_block,
                        register_embedding, register_feed_forward, register_head, register_mixer, register_norm,
                        register_position_encoding)
-from . import norm, rotary, attention, talking_attention, conv_attention, latent_attention, mamba, lightning, chunked_attention, gated_recurrence, time_mix, side_by_side, feed_forward, routed_mlp, block  # noqa: F401  (registers the built-in parts)
+from . import norm, rotary, attention, talking_attention, conv_attention, latent_attention, mamba, lightning, chunked_attention, gated_recurrence, time_mix, side_by_side, diff_attention, mamba2, feed_forward, routed_mlp, block  # noqa: F401  (registers the built-in parts)
 from .model import DecoderModel, Embedding, Head, PairEmbedding
 
 __all__ = ["Block", "FeedForward", "GroupView", "Mixer", "Norm", "PagedKVRequest", "Part", "PendingNorm", "PositionEncoding",

@@ -138,6 +138,12 @@ class ResidualStream:
         self.flush()
         self.x += y.to(self.x.dtype)
 
+    def add_rows_scaled(self, h: torch.Tensor, weights: torch.Tensor, first: int, count: int) -> None:
+        """``x[t] += (sum of weights[t, first : first + count]) * h[t]``: a part's input itself, weighted row by row (experts
+        that return their input).  Comes after the part's ``add_linear``, if it has one."""
+        self.flush()
+        self.ops.add_scaled_rows(self.x, h, weights, first, count)
+
     def launch_deferred(self) -> None:
         """Launch the product that ``add_linear`` left, if any; its sum may stay pending as partial sums."""
         if self.deferred is not None:
@@ -154,6 +160,29 @@ class ResidualStream:
     def value(self) -> torch.Tensor:
         self.flush()
         return self.x
+
+
+class MultiStream:
+    """Several 32-bit residual streams ``xs [streams, T, width]``, all equal to the embedding at the start.  A branch reads a
+    weighted sum of them and is written back into all of them at once (``parts/block.py``, the multi-stream block); the
+    model's output is their sum."""
+
+    def __init__(self, x: torch.Tensor, streams: int, ops):
+        self.ops = ops
+        self.xs = x.new_empty((streams,) + tuple(x.shape))
+        self.xs[:] = x
+
+    def read(self, w_in: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> ResidualStream:
+        """``sum_s w_in[s] x_s`` (None: the plain sum), of the ``rows`` if given, as a stream of its own."""
+        return ResidualStream(self.ops.streams_read(self.xs, w_in, rows), self.ops)
+
+    def write(self, sums: torch.Tensor, bias: Optional[torch.Tensor], mix: torch.Tensor, w_out: torch.Tensor) -> None:
+        """All streams at once from the old ones: ``x_t = sum_s mix[s, t] x_s + w_out[t] (sum(sums) + bias)``; ``sums``
+        float32 ``[P, T, width]`` are the partial sums of a branch's last product."""
+        self.ops.streams_write(self.xs, sums, bias, mix, w_out)
+
+    def value(self) -> torch.Tensor:
+        return self.read(None).x
 
 
 class PendingNorm:

@@ -1,31 +1,36 @@
 """Arrangements of parts in a block.  Post-norm: the branches read the stream itself and are normed on their way out,
 ``x += post(mixer(x)); x += post(feed_forward(x))``.  Parallel: one norm feeds both branches, ``x += mixer(norm(x)) + feed_forward(norm(x))``.
-Sandwich: a norm before and one after each branch,
+Multi-stream: pre-norm over several residual streams, a branch reading ``sum_s in[s] x_s`` and written back as
+``x_t = sum_s mix[s, t] x_s + out[t] y``.  Sandwich: a norm before and one after each branch,
 ``x += post(mixer(pre(x))); x += post(feed_forward(pre(x)))``.  Pre-norm (``crates/mach-model/src/batched.rs:3180-3200,
 4031, 4050, 4453``): ``x += mixer(norm(x)); x += feed_forward(norm(x))``."""
 from __future__ import annotations
 
-from .base import Block
+from .base import Block, MultiStream, Part, TensorDecl
 from .registry import FEED_FORWARDS, MIXERS, NORMS, register_block
 
 
 @register_block("prenorm")
 class PreNormBlock(Block):
-    """Reads ``mixer``, ``feed_forward``, ``mixer_norm`` and ``feed_forward_norm`` of its layer's spec."""
+    """Reads ``mixer``, ``feed_forward`` (may be None, then its norm too), ``mixer_norm`` and ``feed_forward_norm`` of its
+    layer's spec."""
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         self.mixer = MIXERS.build(spec.mixer, rt)
-        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
         self.mixer_norm = NORMS.build(spec.mixer_norm, rt)
-        self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, rt)
+        self.feed_forward = self.feed_forward_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+            self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, rt)
 
     def parts(self):
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        return [self.mixer_norm, self.mixer] + ([self.feed_forward_norm, self.feed_forward] if self.feed_forward is not None else [])
 
     def forward(self, stream, ctx):
         self.mixer.forward(self._input(self.mixer_norm, self.mixer, stream), stream, ctx)
-        self.feed_forward.forward(self._input(self.feed_forward_norm, self.feed_forward, stream), stream, ctx)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(self._input(self.feed_forward_norm, self.feed_forward, stream), stream, ctx)
 
     @staticmethod
     def _input(norm, reader, stream):
@@ -69,6 +74,7 @@ class _Branch:
         self.bias = None
         self.tensor = None
         self.branches = None
+        self.scaled = None
 
     def add_linear(self, a, w, bias=None) -> None:
         self.product, self.bias = (a, w), bias
@@ -78,6 +84,71 @@ class _Branch:
 
     def add(self, y) -> None:
         self.tensor = y
+
+    def add_rows_scaled(self, h, weights, first, count) -> None:
+        self.scaled = (h, weights, first, count)
+
+
+class StreamMix(Part):
+    """The three small tensors with which one branch reads and writes several streams."""
+
+    def tensor_decls(self):
+        n = self.spec.streams
+        return [TensorDecl("in", (n,), "vector"), TensorDecl("out", (n,), "vector"), TensorDecl("mix", (n, n), "vector")]
+
+    def load(self, t):
+        self.w_in, self.w_out, self.w_mix = t["in"], t["out"], t["mix"]
+
+
+@register_block("multistream")
+class MultiStreamBlock(Block):
+    """Pre-norm over several residual streams (``base.MultiStream``).  Reads ``mixer``, ``feed_forward`` (may be None),
+    ``mixer_norm``, ``feed_forward_norm``, ``mixer_streams`` and ``feed_forward_streams`` of its layer's spec.  A branch's
+    input is the norm of ``sum_s in[s] x_s`` (one kernel for the sum and an RMS norm); what it leaves (the operands of a
+    last product, a bias, a finished tensor, rows of its input to be added with weights) is written into all streams by
+    one kernel that also adds the product's partial sums up."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, rt)
+        self.mixer_streams = StreamMix(spec.mixer_streams, rt)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_streams = None
+        if spec.feed_forward is not None:
+            self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+            self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, rt)
+            self.feed_forward_streams = StreamMix(spec.feed_forward_streams, rt)
+
+    def parts(self):
+        out = [self.mixer_norm, self.mixer, self.mixer_streams]
+        if self.feed_forward is not None:
+            out += [self.feed_forward_norm, self.feed_forward, self.feed_forward_streams]
+        return out
+
+    def forward(self, stream, ctx):
+        if not isinstance(stream, MultiStream):
+            raise TypeError("a multi-stream block in a model of one residual stream: the model's spec names no streams")
+        self._branch(self.mixer_norm, self.mixer, self.mixer_streams, stream, ctx)
+        if self.feed_forward is not None:
+            self._branch(self.feed_forward_norm, self.feed_forward, self.feed_forward_streams, stream, ctx)
+
+    def _branch(self, norm, part, mix, stream, ctx):
+        ops = self.rt.ops
+        if type(norm).__name__ == "RMSNorm" and hasattr(ops, "streams_read_norm"):
+            h = ops.streams_read_norm(stream.xs, mix.w_in, norm.weight, norm.spec.eps)
+        else:
+            h = norm.forward(stream.read(mix.w_in))
+        out = _Branch(ops)
+        part.forward(h, out, ctx)
+        if out.product is not None:
+            sums = ops.linear_split(*out.product)
+        elif out.tensor is not None:
+            sums = out.tensor.float().contiguous().unsqueeze(0)
+        else:
+            raise ValueError(f"{type(part).__name__} left neither a last product nor a finished tensor")
+        if out.scaled is not None:  # into the first of the sums, which nobody else holds
+            ops.add_scaled_rows(sums[0], *out.scaled)
+        stream.write(sums, out.bias, mix.w_mix, mix.w_out)
 
 
 @register_block("sandwich")

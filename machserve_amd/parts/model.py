@@ -10,7 +10,7 @@ from typing import List, Optional
 import torch
 
 from ..config.specs import ModelSpec
-from .base import Block, Part, ResidualStream, Runtime, StepContext, TensorDecl, require_kernel_sizes
+from .base import Block, MultiStream, Part, ResidualStream, Runtime, StepContext, TensorDecl, require_kernel_sizes
 from .registry import BLOCKS, EMBEDDINGS, HEADS, NORMS, register_embedding, register_head
 
 
@@ -182,7 +182,8 @@ class DecoderModel:
         ctx.shared.clear()
         embedding = self.embedding
         x = embedding.forward_step(ctx) if getattr(embedding, "reads_step", False) else embedding.forward(ctx.tokens)
-        stream = ResidualStream(x, self.rt.ops)
+        streams = getattr(self.spec, "streams", None)  # several residual streams that all start as the embedding
+        stream = MultiStream(x, streams, self.rt.ops) if streams else ResidualStream(x, self.rt.ops)
         watch = self.observer
         if watch is not None:
             watch("embedding", stream.value())
@@ -194,4 +195,6 @@ class DecoderModel:
                 watch(f"layer{p:02d}", stream.value())
         if ctx.want_rows.numel() == 0:
             return None
+        if streams:  # the sum of the streams, of the wanted rows only
+            return self.head.forward(self.final_norm.forward(stream.read(None, ctx.want_rows)))
         return self.head.forward(self.final_norm.forward(stream, rows=ctx.want_rows))

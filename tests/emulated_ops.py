@@ -197,24 +197,34 @@ class EmulatedOps:
         u, v = x[..., 0::2], x[..., 1::2]
         return torch.stack([u * c - v * sn, v * c + u * sn], -1).flatten(-2)
 
+    @staticmethod
+    def _rotate_halves(x, positions, inv_freq, factor):
+        """``x [T, ..., rot]``: pairs (i, i + rot / 2) rotated by ``positions * inv_freq[i]``."""
+        ang = positions.float().reshape([-1] + [1] * (x.dim() - 1)) * inv_freq.float()
+        c, sn = torch.cos(ang) * factor, torch.sin(ang) * factor
+        half = x.shape[-1] // 2
+        u, v = x[..., :half], x[..., half:]
+        return torch.cat([u * c - v * sn, v * c + u * sn], -1)
+
     def latent_rows(self, proj, q_norm, c_norm, eps, positions, inv_freq, cs_factor, slot_map, kpool, vpool, q_rank, rank, rot,
-                    page_size):
+                    page_size, halves=False):
         row = proj.sum(0) if proj.dim() == 3 else proj
         T = row.shape[0]
         rms = lambda x: x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
         cq = torch.zeros(T, -(-q_rank // 8) * 8)
-        cq[:, :q_rank] = rms(row[:, :q_rank]) * q_norm
+        if q_rank:
+            cq[:, :q_rank] = rms(row[:, :q_rank]) * q_norm
         if c_norm is not None:
             c = self._r(rms(row[:, q_rank:q_rank + rank]) * c_norm)
             page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
             kpool[page, 0, off, :rank] = c
             vpool[page, 0, :rank, off] = c
             if rot:
-                kpool[page, 0, off, rank:rank + rot] = self._r(self._rotate_neighbours(row[:, q_rank + rank:q_rank + rank + rot], positions,
-                                                                                       inv_freq, cs_factor))
-        return self._r(cq)
+                turn = self._rotate_halves if halves else self._rotate_neighbours
+                kpool[page, 0, off, rank:rank + rot] = self._r(turn(row[:, q_rank + rank:q_rank + rank + rot], positions, inv_freq, cs_factor))
+        return self._r(cq) if q_rank else None
 
-    def latent_query(self, q, positions, inv_freq, cs_factor, H, d, rot, rank, hd):
+    def latent_query(self, q, positions, inv_freq, cs_factor, H, d, rot, rank, hd, halves=False):
         T = q.shape[0]
         qh = q.view(T, H, d + rot)
         plain = torch.zeros(T, H, -(-d // 8) * 8)
@@ -222,7 +232,7 @@ class EmulatedOps:
         att = torch.full((T, H, hd), float("nan"))  # the first `rank` columns are the per-head product's to fill
         att[..., rank:] = 0.0
         if rot:
-            att[..., rank:rank + rot] = self._rotate_neighbours(qh[..., d:], positions, inv_freq, cs_factor)
+            att[..., rank:rank + rot] = (self._rotate_halves if halves else self._rotate_neighbours)(qh[..., d:], positions, inv_freq, cs_factor)
         return self._r(plain), self._r(att)
 
     def heads_linear(self, a, w, out=None):
@@ -325,8 +335,11 @@ class EmulatedOps:
         return x
 
     # ------------------------------------------------------------------ q, k and v finished from 32-bit rows
-    def finish_rows(self, rows, q_norm, k_norm, eps, positions, inv_freq, rot, neighbours, slot_map, kpool, vpool, H, KV, d, dv, page_size):
+    def finish_rows(self, rows, q_norm, k_norm, eps, positions, inv_freq, rot, neighbours, slot_map, kpool, vpool, H, KV, d, dv, page_size,
+                    queries_only=False):
         T, dp = rows.shape[0], kpool.shape[3]
+        if queries_only:  # the layer reads another layer's keys and values and writes none
+            KV = 0
         nq, nk = H * d, KV * d
         q, k, v = rows[:, :nq], rows[:, nq:nq + nk], rows[:, nq + nk:nq + nk + KV * dv]
         rms = lambda y: y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps))
@@ -433,25 +446,98 @@ class EmulatedOps:
     def route_limits(self):
         return {"experts": 1024, "top": 64}
 
-    def route(self, h, w, bias, top):
+    def route(self, h, w, bias, top, correction=None, softmax_all=False):
         z = h.float() @ w.t()
         if bias is not None:
             z = z + bias
+        if softmax_all:  # scores over every output; a correction for the choice only; the chosen scores over their sum
+            score = torch.softmax(z, -1)
+            pick = score if correction is None else score + correction
+            idx = torch.topk(pick, top, dim=-1).indices
+            val = torch.gather(score, 1, idx)
+            gates = torch.zeros_like(z)
+            gates.scatter_(1, idx, val / (val.sum(-1, keepdim=True) + 1e-20))
+            return gates
         val, idx = torch.topk(z, top, dim=-1)
         gates = torch.zeros_like(z)
         gates.scatter_(1, idx, torch.softmax(val, -1))
         return gates
 
-    def expert_act(self, up, gates, ff, activation):
+    def expert_act(self, up, gates, ff, activation, experts=None, gated=False):
         T, n = up.shape
-        E = gates.shape[1]
+        E = gates.shape[1] if experts is None else experts
+        mul = None
+        if gated:  # the first half of the columns are the gates, the second the up projections
+            n //= 2
+            up, mul = up[:, :n], up[:, n:]
         if activation == "gelu":
             a = 0.5 * up * (1.0 + torch.erf(up * 0.7071067811865476))
         else:
             a = _act(up, activation)
+        if mul is not None:
+            a = a * mul
         wgt = torch.ones(T, n)
-        wgt[:, :E * ff] = gates.repeat_interleave(ff, dim=1)
+        wgt[:, :E * ff] = gates[:, :E].repeat_interleave(ff, dim=1)
         return self._r(torch.where(wgt != 0, a * wgt, torch.zeros(())))
+
+    def add_scaled_rows(self, x, h, weights, first, count):
+        x += weights[:, first:first + count].sum(-1, keepdim=True) * h.float()
+
+    # ------------------------------------------------------------------ several residual streams
+    def streams_read(self, xs, w_in, rows=None):
+        src = xs if rows is None else xs[:, rows.long()]
+        return src.sum(0) if w_in is None else torch.einsum("s,stw->tw", w_in, src)
+
+    def streams_read_norm(self, xs, w_in, norm_w, eps):
+        u = self.streams_read(xs, w_in)
+        return self._r(u * (1.0 / torch.sqrt((u * u).sum(-1, keepdim=True) / u.shape[-1] + eps)) * norm_w)
+
+    def streams_write(self, xs, sums, bias, mix, w_out):
+        y = sums.sum(0)
+        if bias is not None:
+            y = y + bias
+        xs.copy_(torch.einsum("st,snw->tnw", mix, xs) + w_out[:, None, None] * y[None])
+
+    # ------------------------------------------------------------------ differential attention, state-space duality
+    def sigmoid_rows(self, sums):
+        return torch.sigmoid(sums)
+
+    def diff_combine(self, o, gate, lam, eps, factor, H, KV, hd, dv, out_cols):
+        T, per = o.shape[0], H // KV
+        maps = o.float().view(T, KV, 2, per, hd)[..., :dv]  # (key/value head, map, head of the group)
+        d = (maps[:, :, 0] - lam * maps[:, :, 1]).reshape(T, H, dv)
+        d = d * (1.0 / torch.sqrt((d * d).sum(-1, keepdim=True) / dv + eps)) * factor
+        y = torch.zeros(T, out_cols)
+        y[:, :H * dv] = d.reshape(T, H * dv) * torch.sigmoid(gate)
+        return self._r(y)
+
+    def ssd_limits(self):
+        return {"states": 256, "head_dim": 256}
+
+    def ssd_scan(self, xbc, proj, dt_col, dt_bias, a_log, d_skip, state, seq_q_start, seq_q_len, seq_slot, H, P, N, G):
+        T = xbc.shape[0]
+        act = xbc / (1.0 + torch.exp(-xbc))
+        x, B, C = act[:, :H * P].view(T, H, P), act[:, H * P:H * P + G * N].view(T, G, N), act[:, H * P + G * N:].view(T, G, N)
+        dt = torch.nn.functional.softplus(proj[:, dt_col:dt_col + H] + dt_bias, threshold=30.0)
+        decay = torch.exp(-torch.exp(a_log) * dt)
+        group = torch.arange(H) // (H // G)
+        y = torch.zeros(T, H, P)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            S = state[slot].clone()
+            for t in range(q0, q0 + n):
+                S = decay[t][:, None, None] * S + dt[t][:, None, None] * B[t][group][:, :, None] * x[t][:, None, :]
+                y[t] = torch.einsum("hnp,hn->hp", S, C[t][group]) + d_skip[:, None] * x[t]
+            state[slot] = S
+        return y.view(T, H * P)
+
+    def gated_group_norm(self, y, proj, z_col, weight, eps, groups, out_cols):
+        T, n = y.shape
+        z = proj[:, z_col:z_col + n]
+        g = (y * z / (1.0 + torch.exp(-z))).view(T, groups, n // groups)
+        g = g * (1.0 / torch.sqrt((g * g).sum(-1, keepdim=True) / (n // groups) + eps))
+        out = torch.zeros(T, out_cols)
+        out[:, :n] = g.reshape(T, n) * weight
+        return self._r(out)
 
     def softcap(self, logits, scale, cap):
         v = logits * scale
