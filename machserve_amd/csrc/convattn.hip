@@ -393,6 +393,34 @@ __global__ __launch_bounds__(256) void finish_rows_kernel(FinishArgs a) {
     }
 }
 
+// Differential attention behind the attention kernel.  o [T, 2 H maps, dp]: the maps of a key/value head's group lie side
+// by side, (key/value head, map, head of the group).  A head's result is map 0 minus lam times map 1 over its first dv
+// numbers, divided by its root mean square, times `factor`, times sigmoid(gate); heads side by side in rows of ld_out
+// numbers (zeros behind H * dv).  A wave a head.
+__global__ __launch_bounds__(256) void diff_combine_kernel(const elem_t* __restrict__ o, const float* __restrict__ gate,
+                                                           elem_t* __restrict__ out, float lam, float eps, float factor, int H, int KV,
+                                                           int dp, int dv, int ld_out) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63, h = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (blockIdx.y == 0)
+        for (int c = H * dv + threadIdx.x; c < ld_out; c += 256) out[(size_t)t * ld_out + c] = from_f32<elem_t>(0.f);
+    if (h >= H) return;  // the same for the whole wave; no barrier below
+    const int per = H / KV, kvh = h / per, in_group = h - kvh * per;
+    const elem_t* a1 = o + ((size_t)t * 2 * H + (size_t)(kvh * 2) * per + in_group) * dp;
+    const elem_t* a2 = a1 + (size_t)per * dp;
+    float ss = 0.f;
+    for (int e = lane; e < dv; e += 64) {
+        const float v = to_f32(a1[e]) - lam * to_f32(a2[e]);
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float inv = factor / sqrtf(ss / (float)dv + eps);
+    for (int e = lane; e < dv; e += 64) {
+        const float v = to_f32(a1[e]) - lam * to_f32(a2[e]);
+        const float gz = gate[(size_t)t * H * dv + h * dv + e];
+        out[(size_t)t * ld_out + h * dv + e] = from_f32<elem_t>(v * inv / (1.0f + expf(-gz)));
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -434,7 +462,8 @@ extern "C" int ms_conv_rows(const float* proj, int n_partials, int stride, const
 extern "C" int ms_finish_rows(const float* rows, int stride, const float* q_norm, const float* k_norm, float eps, const int* positions,
                               const float* inv_freq, int rot, int neighbours, const int* slot_map, void* q_out, void* kpool, void* vpool,
                               int T, int H, int KV, int d, int dv, int dp, int ps, hipStream_t stream) {
-    MS_REQUIRE(T > 0 && H > 0 && KV > 0 && d > 0 && dv > 0 && dp >= d && dp >= dv, "finish rows: %d rows, %d / %d heads of %d and %d in %d",
+    // KV 0: the rows hold queries only (the layer reads another layer's keys and values); nothing is written to the pools
+    MS_REQUIRE(T > 0 && H > 0 && KV >= 0 && d > 0 && dv > 0 && dp >= d && dp >= dv, "finish rows: %d rows, %d / %d heads of %d and %d in %d",
                T, H, KV, d, dv, dp);
     const int n = H * d + KV * d + KV * dv;
     MS_REQUIRE(stride >= n && n + rot <= CONV_MAX_ROW, "finish rows: a row of %d numbers (stride %d, at most %d)", n, stride, CONV_MAX_ROW);
@@ -443,4 +472,13 @@ extern "C" int ms_finish_rows(const float* rows, int stride, const float* q_norm
                  (elem_t*)vpool, H, KV, d, dv, dp, ps};
     hipLaunchKernelGGL(finish_rows_kernel, dim3(T), dim3(256), (size_t)(stride + rot) * sizeof(float), stream, a);
     return check_launch("finish_rows");
+}
+
+extern "C" int ms_diff_combine(const void* o, const float* gate, void* out, float lam, float eps, float factor, int T, int H, int KV, int dp,
+                               int dv, int ld_out, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && H > 0 && KV > 0 && H % KV == 0 && dv > 0 && dp >= dv && ld_out >= H * dv, "diff_combine: %d rows, %d / %d heads of %d in %d",
+               T, H, KV, dv, dp);
+    hipLaunchKernelGGL(diff_combine_kernel, dim3(T, ceil_div(H, 4)), dim3(256), 0, stream, (const elem_t*)o, gate, (elem_t*)out, lam, eps,
+                       factor, H, KV, dp, dv, ld_out);
+    return check_launch("diff_combine");
 }

@@ -35,6 +35,7 @@ struct LatentRowArgs {
     elem_t* kpool;          // [pages, 1, ps, hd]
     elem_t* vpool;          // [pages, 1, hd, ps]
     int q_rank, rank, rot, hd, ps;
+    int halves;             // the key part's pairs are (i, i + rot / 2), not (2i, 2i + 1)
 };
 
 // One block a row.  Columns of the key beyond rank + rot and rows of the value beyond rank are never written: the
@@ -67,9 +68,11 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
     ssq = block_sum<256>(ssq, scratch);
     ssc = block_sum<256>(ssc, scratch);
     __syncthreads();
-    const float inv_q = 1.0f / sqrtf(ssq / (float)a.q_rank + a.eps);
-    for (int c = threadIdx.x; c < a.cq_ld; c += 256)
-        a.cq_out[(size_t)t * a.cq_ld + c] = from_f32<elem_t>(c < a.q_rank ? row[c] * inv_q * a.q_norm[c] : 0.f);
+    if (a.q_rank > 0) {  // 0: the queries have no bottleneck and are not this kernel's business
+        const float inv_q = 1.0f / sqrtf(ssq / (float)a.q_rank + a.eps);
+        for (int c = threadIdx.x; c < a.cq_ld; c += 256)
+            a.cq_out[(size_t)t * a.cq_ld + c] = from_f32<elem_t>(c < a.q_rank ? row[c] * inv_q * a.q_norm[c] : 0.f);
+    }
     if (!kv) return;
     const int slot = a.slot_map[t];
     if (slot < 0) return;
@@ -89,9 +92,10 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
         sincosf(pos * a.inv_freq[i], &sn, &cs);
         sn *= a.cs_factor;
         cs *= a.cs_factor;
-        const float u = kr[2 * i], v = kr[2 * i + 1];
-        krow[a.rank + 2 * i] = from_f32<elem_t>(u * cs - v * sn);
-        krow[a.rank + 2 * i + 1] = from_f32<elem_t>(v * cs + u * sn);
+        const int iu = a.halves ? i : 2 * i, iv = a.halves ? i + a.rot / 2 : 2 * i + 1;
+        const float u = kr[iu], v = kr[iv];
+        krow[a.rank + iu] = from_f32<elem_t>(u * cs - v * sn);
+        krow[a.rank + iv] = from_f32<elem_t>(v * cs + u * sn);
     }
 }
 
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
 __global__ __launch_bounds__(256) void latent_query_kernel(const float* __restrict__ q, const int* __restrict__ positions,
                                                            const float* __restrict__ inv_freq, float cs_factor,
                                                            elem_t* __restrict__ plain, elem_t* __restrict__ att, int H, int d, int dp,
-                                                           int rot, int rank, int hd) {
+                                                           int rot, int rank, int hd, int halves) {
     const int t = blockIdx.x;
     const float pos = (float)positions[t];
     const float* qr = q + (size_t)t * H * (d + rot);
@@ -118,9 +122,10 @@ __global__ __launch_bounds__(256) void latent_query_kernel(const float* __restri
             sincosf(pos * inv_freq[i], &sn, &cs);
             sn *= cs_factor;
             cs *= cs_factor;
-            const float u = qr[h * (d + rot) + d + 2 * i], v = qr[h * (d + rot) + d + 2 * i + 1];
-            dst[2 * i] = from_f32<elem_t>(u * cs - v * sn);
-            dst[2 * i + 1] = from_f32<elem_t>(v * cs + u * sn);
+            const int iu = halves ? i : 2 * i, iv = halves ? i + half : 2 * i + 1;
+            const float u = qr[h * (d + rot) + d + iu], v = qr[h * (d + rot) + d + iv];
+            dst[iu] = from_f32<elem_t>(u * cs - v * sn);
+            dst[iv] = from_f32<elem_t>(v * cs + u * sn);
         } else {
             dst[rot + (i - half)] = from_f32<elem_t>(0.f);
         }
@@ -190,6 +195,11 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(HeadsLinearArgs g) {
         }
 }
 
+// out[i] = sigmoid(in[i]): a gate per row and head from 32-bit sums
+__global__ __launch_bounds__(256) void sigmoid_rows_kernel(const float* __restrict__ in, float* __restrict__ out, long n) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) out[i] = 1.0f / (1.0f + expf(-in[i]));
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -201,8 +211,10 @@ extern "C" int ms_latent_max_row() { return LATENT_MAX_ROW; }
 // layer's cache); then slot_map, kpool, vpool, inv_freq are not read.
 extern "C" int ms_latent_rows(const float* proj, int n_partials, int stride, const float* q_norm, const float* c_norm, float eps,
                               const int* positions, const float* inv_freq, float cs_factor, const int* slot_map, void* cq_out,
-                              int cq_ld, void* kpool, void* vpool, int T, int q_rank, int rank, int rot, int hd, int ps, hipStream_t stream) {
-    MS_REQUIRE(T > 0 && n_partials >= 1 && q_rank > 0 && cq_ld >= q_rank, "latent rows: %d rows, %d partial sums, query latent of %d in %d", T, n_partials, q_rank, cq_ld);
+                              int cq_ld, void* kpool, void* vpool, int T, int q_rank, int rank, int rot, int hd, int ps, int halves,
+                              hipStream_t stream) {
+    MS_REQUIRE(T > 0 && n_partials >= 1 && q_rank >= 0 && cq_ld >= q_rank, "latent rows: %d rows, %d partial sums, query latent of %d in %d", T, n_partials, q_rank, cq_ld);
+    MS_REQUIRE(q_rank > 0 || c_norm, "latent rows: neither a query latent nor a cache to write");
     const int n = q_rank + (c_norm ? rank + rot : 0);
     MS_REQUIRE(stride >= n && n <= LATENT_MAX_ROW, "latent rows: a row of %d numbers (stride %d, at most %d)", n, stride, LATENT_MAX_ROW);
     if (c_norm) {
@@ -210,17 +222,17 @@ extern "C" int ms_latent_rows(const float* proj, int n_partials, int stride, con
         MS_REQUIRE(positions && slot_map && kpool && vpool && (rot == 0 || inv_freq), "latent rows: the layer writes the cache");
     }
     LatentRowArgs a{proj, n_partials, (size_t)T * stride, stride, q_norm, c_norm, eps, positions, inv_freq, cs_factor, slot_map,
-                    (elem_t*)cq_out, cq_ld, (elem_t*)kpool, (elem_t*)vpool, q_rank, rank, rot, hd, ps};
+                    (elem_t*)cq_out, cq_ld, (elem_t*)kpool, (elem_t*)vpool, q_rank, rank, rot, hd, ps, halves};
     hipLaunchKernelGGL(latent_row_kernel, dim3(T), dim3(256), (size_t)n * sizeof(float), stream, a);
     return check_launch("latent_rows");
 }
 
 extern "C" int ms_latent_query(const float* q, const int* positions, const float* inv_freq, float cs_factor, void* plain, void* att,
-                               int T, int H, int d, int dp, int rot, int rank, int hd, hipStream_t stream) {
+                               int T, int H, int d, int dp, int rot, int rank, int hd, int halves, hipStream_t stream) {
     MS_REQUIRE(T > 0 && H > 0 && d > 0 && dp >= d, "latent query: %d rows, %d heads, plain part %d in %d", T, H, d, dp);
     MS_REQUIRE(rot >= 0 && rot % 2 == 0 && rank + rot <= hd && (rot == 0 || inv_freq), "latent query: latent %d + rotated part %d in a key of %d", rank, rot, hd);
     hipLaunchKernelGGL(latent_query_kernel, dim3(T), dim3(256), 0, stream, q, positions, inv_freq, cs_factor, (elem_t*)plain,
-                       (elem_t*)att, H, d, dp, rot, rank, hd);
+                       (elem_t*)att, H, d, dp, rot, rank, hd, halves);
     return check_launch("latent_query");
 }
 
@@ -239,4 +251,10 @@ extern "C" int ms_heads_linear(const void* a, long lda, long a_head, const void*
         hipLaunchKernelGGL((heads_linear_kernel<1, 1, false>), dim3(1, ceil_div(N, 64), B), dim3(256), 0, stream, g);
     }
     return check_launch("heads_linear");
+}
+
+extern "C" int ms_sigmoid_rows(const float* in, float* out, long n, hipStream_t stream) {
+    MS_REQUIRE(n > 0 && in && out, "sigmoid_rows: %ld numbers", n);
+    hipLaunchKernelGGL(sigmoid_rows_kernel, dim3((unsigned)std::min<long>(ceil_div(n, 256L), 4096L)), dim3(256), 0, stream, in, out, n);
+    return check_launch("sigmoid_rows");
 }

@@ -5,7 +5,8 @@ embedding, sampling), one attention library per element type and head-size tile,
 library per element type for the mixers with state of fixed size ("recurrent"), for the
 attention whose heads exchange scores ("talking"), for attention through a latent ("latent") and for
 attention behind a short convolution ("convattn"), for linear recurrences with gates that depend on the token
-("linrec") and for feed-forwards of routed experts ("routed"), which only the models that have them load.  A
+("linrec"), for feed-forwards of routed experts ("routed"), for several residual streams ("multistream") and for the
+state-space duality layer ("ssd"), which only the models that have them load.  A
 library is rebuilt when the hash of its sources and flags differs from the stamp beside it,
 so a fresh checkout compiles at its first call exactly the libraries the model at hand
 needs, and prints a line now and then while it does.
@@ -69,7 +70,7 @@ def _hipcc() -> str:
 
 
 EXTRA_KINDS = {"recurrent": "recurrent.hip", "talking": "talking.hip", "latent": "latent.hip", "convattn": "convattn.hip",
-               "linrec": "linrec.hip", "routed": "routed.hip"}  # libraries that only some models load
+               "linrec": "linrec.hip", "routed": "routed.hip", "multistream": "multistream.hip", "ssd": "ssd.hip"}  # libraries that only some models load
 
 
 def _sources_of(kind: str):

@@ -852,18 +852,22 @@ class HipOps:
 
     def latent_rows(self, proj: torch.Tensor, q_norm: torch.Tensor, c_norm: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
                     inv_freq: Optional[torch.Tensor], cs_factor: float, slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
-                    vpool: Optional[torch.Tensor], q_rank: int, rank: int, rot: int, page_size: int) -> torch.Tensor:
+                    vpool: Optional[torch.Tensor], q_rank: int, rank: int, rot: int, page_size: int, halves: bool = False) -> Optional[torch.Tensor]:
         """Finishes the rows of the down projections given as float32 partial sums ``[P, T, stride]`` (query latent
         ``[q_rank]``, then, if the layer writes a cache (``c_norm`` given), latent ``[rank]`` and key part ``[rot]``): RMS
         norm with weight of the query latent, returned ``[T, q_rank up to a multiple of 8]`` in the element type (zeros behind); RMS norm with weight of the
         latent, written as columns ``0 .. rank`` of the row's key and as the row's value; the key part rotated in pairs
-        ``(2i, 2i + 1)`` by ``positions * inv_freq`` with cosines and sines times ``cs_factor``, written behind it."""
+        ``(2i, 2i + 1)`` (with ``halves``: ``(i, i + rot / 2)``) by ``positions * inv_freq`` with cosines and sines times
+        ``cs_factor``, written behind it.  ``q_rank`` 0: the rows hold no query latent, and nothing is returned."""
         lib = self._extra_lib("latent")
         if proj.dim() == 2:
             proj = proj.unsqueeze(0)
         P, T, stride = proj.shape
         self._want(proj, torch.float32, "latent rows")
-        self._want(q_norm, torch.float32, "query latent norm weight", q_rank)
+        if q_rank:
+            self._want(q_norm, torch.float32, "query latent norm weight", q_rank)
+        elif c_norm is None:
+            raise KernelError("latent rows: neither a query latent nor a cache to write")
         hd = 0
         if c_norm is not None:
             self._want(c_norm, torch.float32, "latent norm weight", rank)
@@ -874,15 +878,15 @@ class HipOps:
             pages, _, _, hd = kpool.shape
             self._want(kpool, self.dtype, "latent key pool", pages, 1, page_size, hd)
             self._want(vpool, self.dtype, "latent value pool", pages, 1, hd, page_size)
-        cq = torch.empty((T, -(-q_rank // 8) * 8), dtype=self.dtype, device=proj.device)
+        cq = torch.empty((T, -(-q_rank // 8) * 8), dtype=self.dtype, device=proj.device) if q_rank else None
         self._check(lib, lib.ms_latent_rows(_ptr(proj), _c_int(P), _c_int(stride), _ptr(q_norm), _ptr(c_norm), _c_float(eps),
                                             _ptr(positions), _ptr(inv_freq), _c_float(cs_factor), _ptr(slot_map), _ptr(cq),
-                                            _c_int(cq.shape[1]), _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(q_rank), _c_int(rank), _c_int(rot), _c_int(hd),
-                                            _c_int(page_size), self._stream()))
+                                            _c_int(cq.shape[1] if q_rank else 0), _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(q_rank), _c_int(rank), _c_int(rot), _c_int(hd),
+                                            _c_int(page_size), _c_int(int(halves)), self._stream()))
         return cq
 
     def latent_query(self, q: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], cs_factor: float, H: int, d: int,
-                     rot: int, rank: int, hd: int):
+                     rot: int, rank: int, hd: int, halves: bool = False):
         """From the up-projected queries ``q`` float32 ``[T, H * (d + rot)]``: ``(plain [T, H, dp], att [T, H, hd])`` in the
         element type, ``dp`` = ``d`` rounded up to 8.  ``plain`` holds the heads' first ``d`` numbers; ``att``, the queries
         of the attention over the latent cache, has its columns ``rank .. rank + rot`` set to the rotated rest and zeros
@@ -898,8 +902,16 @@ class HipOps:
         att = torch.empty((T, H, hd), dtype=self.dtype, device=q.device)
         self._check(lib, lib.ms_latent_query(_ptr(q), _ptr(positions), _ptr(inv_freq), _c_float(cs_factor), _ptr(plain), _ptr(att),
                                              _c_int(T), _c_int(H), _c_int(d), _c_int(dp), _c_int(rot), _c_int(rank), _c_int(hd),
-                                             self._stream()))
+                                             _c_int(int(halves)), self._stream()))
         return plain, att
+
+    def sigmoid_rows(self, sums: torch.Tensor) -> torch.Tensor:
+        """``sigmoid(sums)`` of float32 sums, float32: a gate per row and head."""
+        lib = self._extra_lib("latent")
+        self._want(sums, torch.float32, "gate sums")
+        out = torch.empty_like(sums)
+        self._check(lib, lib.ms_sigmoid_rows(_ptr(sums), _ptr(out), ctypes.c_long(sums.numel()), self._stream()))
+        return out
 
     def heads_linear(self, a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A product per head: ``out[t, b, :N] = w[b] @ a[t, b, :]`` for ``a [T, B, K]`` and ``w [B, N, K]``.  ``out``
@@ -1030,8 +1042,10 @@ class HipOps:
     # ------------------------------------------------------------------ q, k and v finished from 32-bit rows
     def finish_rows(self, rows: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
                     positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot: int, neighbours: bool, slot_map: torch.Tensor,
-                    kpool: torch.Tensor, vpool: torch.Tensor, H: int, KV: int, d: int, dv: int, page_size: int) -> torch.Tensor:
-        """``rows`` float32 ``[T, >= H d + KV d + KV dv]`` hold q, k and v: an RMS norm over all of q and one over all of k
+                    kpool: torch.Tensor, vpool: torch.Tensor, H: int, KV: int, d: int, dv: int, page_size: int,
+                    queries_only: bool = False) -> torch.Tensor:
+        """``queries_only``: the rows hold q alone and nothing is written to the pools, which belong to another layer.
+        ``rows`` float32 ``[T, >= H d + KV d + KV dv]`` hold q, k and v: an RMS norm over all of q and one over all of k
         (weights; None: none), the rotation of the first ``rot`` numbers of every head of q and k by ``position * inv_freq``
         (pairs of neighbours, or ``(i, i + rot / 2)``), k and v written into their pages.  Returns q ``[T, H * dp]`` in the
         element type, ``dp`` the pools' head size (zeros beyond ``d``)."""
@@ -1054,9 +1068,24 @@ class HipOps:
         q = torch.empty((T, H * dp), dtype=self.dtype, device=rows.device)
         self._check(lib, lib.ms_finish_rows(_ptr(rows), _c_int(stride), _ptr(q_norm), _ptr(k_norm), _c_float(eps), _ptr(positions),
                                             _ptr(inv_freq), _c_int(rot), _c_int(int(neighbours)), _ptr(slot_map), _ptr(q), _ptr(kpool),
-                                            _ptr(vpool), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(dp),
+                                            _ptr(vpool), _c_int(T), _c_int(H), _c_int(0 if queries_only else KV), _c_int(d), _c_int(dv), _c_int(dp),
                                             _c_int(page_size), self._stream()))
         return q
+
+    def diff_combine(self, o: torch.Tensor, gate: torch.Tensor, lam: float, eps: float, factor: float, H: int, KV: int, hd: int, dv: int,
+                     out_cols: int) -> torch.Tensor:
+        """Differential attention behind the attention kernel.  ``o [T, 2 H hd]`` in the element type holds two maps a head,
+        ordered (key/value head, map, head of the group); a head's result is ``map0 - lam map1`` over its first ``dv``
+        numbers, divided by its root mean square (``eps``), times ``factor`` and ``sigmoid(gate)`` (float32 ``[T, H dv]``).
+        Heads side by side, ``[T, out_cols]`` in the element type with zeros behind ``H dv``."""
+        lib = self._extra_lib("convattn")
+        T = o.shape[0]
+        self._want(o, self.dtype, "diff_combine maps", T, 2 * H * hd)
+        self._want(gate, torch.float32, "diff_combine gate", T, H * dv)
+        out = torch.empty((T, out_cols), dtype=self.dtype, device=o.device)
+        self._check(lib, lib.ms_diff_combine(_ptr(o), _ptr(gate), _ptr(out), _c_float(lam), _c_float(eps), _c_float(factor), _c_int(T), _c_int(H),
+                                             _c_int(KV), _c_int(hd), _c_int(dv), _c_int(out_cols), self._stream()))
+        return out
 
     # ------------------------------------------------------------------ linear recurrences with gates that depend on the token
     def linrec_limits(self) -> dict:
@@ -1206,9 +1235,12 @@ class HipOps:
     def route_limits(self) -> dict:
         return {"experts": self._extra_lib("routed").ms_route_max_experts(), "top": 64}
 
-    def route(self, h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], top: int) -> torch.Tensor:
+    def route(self, h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], top: int, correction: Optional[torch.Tensor] = None,
+              softmax_all: bool = False) -> torch.Tensor:
         """Float32 ``[T, experts]``: for every row its weight for each expert, the softmax over the ``top`` largest of the
-        logits ``h @ w.T + bias`` (32-bit sums, float32 weights; the lower index wins a tie), zero for the others."""
+        logits ``h @ w.T + bias`` (32-bit sums, float32 weights; the lower index wins a tie), zero for the others.  With
+        ``softmax_all`` the scores are the softmax over all logits, the ``top`` largest of score + ``correction`` are chosen,
+        and the weights are the chosen scores over their sum (+ 1e-20)."""
         lib = self._extra_lib("routed")
         T, d = h.shape
         E = w.shape[0]
@@ -1216,23 +1248,140 @@ class HipOps:
         self._want(w, torch.float32, "route weight", E, d)
         if bias is not None:
             self._want(bias, torch.float32, "route bias", E)
+        if correction is not None:
+            self._want(correction, torch.float32, "route correction", E)
         gates = torch.empty((T, E), dtype=torch.float32, device=h.device)
-        self._check(lib, lib.ms_route(_ptr(h), _ptr(w), _ptr(bias), _ptr(gates), _c_int(T), _c_int(d), _c_int(E), _c_int(top), self._stream()))
+        self._check(lib, lib.ms_route(_ptr(h), _ptr(w), _ptr(bias), _ptr(gates), _c_int(T), _c_int(d), _c_int(E), _c_int(top),
+                                      _c_int(int(softmax_all)), _ptr(correction), self._stream()))
         return gates
 
-    def expert_act(self, up: torch.Tensor, gates: torch.Tensor, ff: int, activation: str) -> torch.Tensor:
+    def expert_act(self, up: torch.Tensor, gates: torch.Tensor, ff: int, activation: str, experts: Optional[int] = None,
+                   gated: bool = False) -> torch.Tensor:
         """``act(up[t, c]) * gates[t, c // ff]`` in the element type for float32 ``up [T, n]``; the columns beyond
-        ``experts * ff`` (an expert every row uses) carry weight one."""
+        ``experts * ff`` (an expert every row uses) carry weight one.  ``experts``: how many of the gates' columns are
+        experts with columns here (None: all).  ``gated``: ``up`` is ``[T, 2 n]``, the experts' gates and then their up
+        projections, and the result ``act(gate) * up * weight``."""
         lib = self._extra_lib("routed")
         T, n = up.shape
-        E = gates.shape[1]
+        if gated:
+            if n % 2:
+                raise KernelError(f"experts: {n} columns are not gates and up projections")
+            n //= 2
+        E = gates.shape[1] if experts is None else experts
         self._want(up, torch.float32, "expert sums")
-        self._want(gates, torch.float32, "expert weights", T, E)
+        self._want(gates, torch.float32, "expert weights", T, gates.shape[1])
+        if E > gates.shape[1]:
+            raise KernelError(f"experts: {E} experts for weights of {gates.shape[1]} columns")
         if activation not in self.EXPERT_ACTIVATIONS:
             raise KernelError(f"experts: activation {activation!r} is not built (built: {', '.join(sorted(self.EXPERT_ACTIVATIONS))})")
         out = torch.empty((T, n), dtype=self.dtype, device=up.device)
         self._check(lib, lib.ms_expert_act(_ptr(up), _ptr(gates), _ptr(out), _c_int(T), _c_int(n), _c_int(E), _c_int(ff),
-                                           _c_int(self.EXPERT_ACTIVATIONS[activation]), self._stream()))
+                                           _c_int(self.EXPERT_ACTIVATIONS[activation]), _c_int(gates.shape[1]), _c_int(int(gated)), self._stream()))
+        return out
+
+    def add_scaled_rows(self, x: torch.Tensor, h: torch.Tensor, weights: torch.Tensor, first: int, count: int) -> None:
+        """``x[t] += (sum of weights[t, first : first + count]) * h[t]`` for float32 ``x [T, d]``, ``h`` in the element type and
+        float32 ``weights [T, n]``: rows of a part's own input added with a weight a row."""
+        lib = self._extra_lib("routed")
+        T, d = x.shape
+        self._want(x, torch.float32, "add_scaled_rows sums")
+        self._want(h, self.dtype, "add_scaled_rows rows", T, d)
+        self._want(weights, torch.float32, "add_scaled_rows weights", T, weights.shape[1])
+        self._check(lib, lib.ms_add_scaled_rows(_ptr(x), _ptr(h), _ptr(weights), _c_int(weights.shape[1]), _c_int(first), _c_int(count),
+                                                _c_int(T), _c_int(d), self._stream()))
+
+    # ------------------------------------------------------------------ several residual streams
+    def streams_limits(self) -> dict:
+        lib = self._extra_lib("multistream")
+        return {"streams": lib.ms_streams_max(), "row": lib.ms_streams_max_row()}
+
+    def _streams(self, xs: torch.Tensor):
+        self._want(xs, torch.float32, "streams")
+        if xs.dim() != 3:
+            raise KernelError(f"streams of shape {tuple(xs.shape)}: [streams, rows, width] wanted")
+        return xs.shape
+
+    def streams_read(self, xs: torch.Tensor, w_in: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``sum_s w_in[s] xs[s]`` (None: the plain sum) of float32 ``xs [S, T, d]``, of the ``rows`` if given; float32."""
+        lib = self._extra_lib("multistream")
+        S, T, d = self._streams(xs)
+        if w_in is not None:
+            self._want(w_in, torch.float32, "streams' input weights", S)
+        R = T
+        if rows is not None:
+            self._want(rows, torch.int32, "streams' rows")
+            R = rows.numel()
+        out = torch.empty((R, d), dtype=torch.float32, device=xs.device)
+        self._check(lib, lib.ms_streams_read(_ptr(xs), _ptr(w_in), _ptr(rows), _c_int(R), _ptr(None), _c_float(0.0), _ptr(out), _ptr(None), _c_int(S),
+                                             _c_int(T), _c_int(d), self._stream()))
+        return out
+
+    def streams_read_norm(self, xs: torch.Tensor, w_in: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float) -> torch.Tensor:
+        """``rmsnorm(sum_s w_in[s] xs[s]) * norm_w`` in the element type, one kernel."""
+        lib = self._extra_lib("multistream")
+        S, T, d = self._streams(xs)
+        if w_in is not None:
+            self._want(w_in, torch.float32, "streams' input weights", S)
+        self._want(norm_w, torch.float32, "streams' norm weight", d)
+        out = torch.empty((T, d), dtype=self.dtype, device=xs.device)
+        self._check(lib, lib.ms_streams_read(_ptr(xs), _ptr(w_in), _ptr(None), _c_int(T), _ptr(norm_w), _c_float(eps), _ptr(None), _ptr(out), _c_int(S),
+                                             _c_int(T), _c_int(d), self._stream()))
+        return out
+
+    def streams_write(self, xs: torch.Tensor, sums: torch.Tensor, bias: Optional[torch.Tensor], mix: torch.Tensor, w_out: torch.Tensor) -> None:
+        """In place, all streams at once from the old ones: ``xs[t] = sum_s mix[s, t] xs[s] + w_out[t] (sum(sums) + bias)`` for
+        float32 ``xs [S, T, d]`` and the partial sums ``sums [P, T, d]`` of a branch's last product."""
+        lib = self._extra_lib("multistream")
+        S, T, d = self._streams(xs)
+        self._want(sums, torch.float32, "streams' sums", sums.shape[0], T, d)
+        if bias is not None:
+            self._want(bias, torch.float32, "streams' bias", d)
+        self._want(mix, torch.float32, "streams' mixing matrix", S, S)
+        self._want(w_out, torch.float32, "streams' output weights", S)
+        self._check(lib, lib.ms_streams_write(_ptr(xs), _ptr(sums), _c_int(sums.shape[0]), _ptr(bias), _ptr(mix), _ptr(w_out), _c_int(S),
+                                              _c_int(T), _c_int(d), self._stream()))
+
+    # ------------------------------------------------------------------ state-space duality
+    def ssd_limits(self) -> dict:
+        lib = self._extra_lib("ssd")
+        return {"states": lib.ms_ssd_max_states(), "head_dim": lib.ms_ssd_max_head()}
+
+    def ssd_scan(self, xbc: torch.Tensor, proj: torch.Tensor, dt_col: int, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+                 state: torch.Tensor, seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor, H: int, P: int, N: int,
+                 G: int) -> torch.Tensor:
+        """The recurrence of the second Mamba layer over the step's rows.  ``xbc`` float32 ``[T, H P + 2 G N]``: x, B and C
+        behind their convolution, before their SiLU; ``proj`` float32 ``[T, ld]`` whose columns ``dt_col .. dt_col + H`` are the
+        raw step sizes; ``dt = softplus(raw + dt_bias)``, ``S <- exp(-exp(a_log) dt) S + dt B x^T``, ``y = S^T C + d_skip x``;
+        ``state`` float32 ``[slots, H, N, P]`` is carried on.  Returns float32 ``y [T, H P]``."""
+        lib = self._extra_lib("ssd")
+        T = xbc.shape[0]
+        self._want(xbc, torch.float32, "ssd x, B and C", T, H * P + 2 * G * N)
+        self._want(proj, torch.float32, "ssd projection", T, proj.shape[1])
+        for t, n in ((dt_bias, "dt_bias"), (a_log, "A_log"), (d_skip, "D")):
+            self._want(t, torch.float32, f"ssd {n}", H)
+        self._want(state, torch.float32, "ssd state", state.shape[0], H, N, P)
+        S = self._seq_operands("ssd", seq_q_start, seq_q_len, seq_slot)
+        y = torch.empty((T, H * P), dtype=torch.float32, device=xbc.device)
+        self._check(lib, lib.ms_ssd_scan(_ptr(xbc), _c_int(xbc.shape[1]), _ptr(proj), _c_int(proj.shape[1]), _c_int(dt_col), _ptr(dt_bias),
+                                         _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S),
+                                         _ptr(y), _c_int(T), _c_int(H), _c_int(P), _c_int(N), _c_int(G), self._stream()))
+        return y
+
+    def gated_group_norm(self, y: torch.Tensor, proj: torch.Tensor, z_col: int, weight: torch.Tensor, eps: float, groups: int,
+                         out_cols: int) -> torch.Tensor:
+        """``y * silu(z)`` RMS-normed in ``groups`` equal parts, times ``weight``, in the element type ``[T, out_cols]`` (zeros
+        behind the ``n`` columns of ``y``); ``z`` is columns ``z_col .. z_col + n`` of float32 ``proj``."""
+        lib = self._extra_lib("ssd")
+        T, n = y.shape
+        self._want(y, torch.float32, "gated norm input")
+        self._want(proj, torch.float32, "gated norm gate", T, proj.shape[1])
+        if z_col < 0 or z_col + n > proj.shape[1] or out_cols < n:
+            raise KernelError(f"gated norm: gate columns {z_col}..{z_col + n} of {tuple(proj.shape)}, {out_cols} columns out")
+        self._want(weight, torch.float32, "gated norm weight", n)
+        out = torch.empty((T, out_cols), dtype=self.dtype, device=y.device)
+        z = _c_void(proj.data_ptr() + z_col * 4)
+        self._check(lib, lib.ms_gated_group_norm(_ptr(y), z, _c_int(proj.shape[1]), _ptr(weight), _ptr(out), _c_int(out_cols), _c_int(T),
+                                                 _c_int(n), _c_int(groups), _c_float(eps), self._stream()))
         return out
 
     # ------------------------------------------------------------------ sampling
