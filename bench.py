@@ -338,6 +338,30 @@ def melerax_configs(z):
     return (melerax,) + design_configs(z)
 
 
+def befirax_configs(z):
+    """(Befirax, Melerax, Qwen2) configurations of one size.  Befirax over two residual streams: the state-space duality
+    layer (twice the width inside, heads of 64, 128 states), differential attention behind a convolution with half the
+    heads, each of two maps (as many query and key maps of the head size as the other designs have heads, values once per
+    key/value head), latent attention under the other designs' window (a latent of 192 beside a rotated part of 64), and
+    differential attention that reads the second layer's keys and values; every feed-forward 8 gated experts of half
+    the dense size, 2 a token, and one expert that returns its input (a token uses as many weights as in the dense
+    feed-forward)."""
+    w, H, kv, hd = z["width"], z["heads"], z["kv"], z["hd"]
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2}, "router": {"experts": 8, "top": 2, "identity": 1}}
+    att = {"heads": H // 2, "kv_heads": max(kv // 2, 1), "dim": hd, "vdim": hd, "scale": hd ** -0.5, "diff": 0.3, "conv": 4,
+           "rot": {"base": 10000.0, "dims": hd // 2}}
+    lat = {"heads": H, "dim": hd, "rot_dim": 64, "vdim": hd, "kv_rank": 192, "scale": (hd + 64) ** -0.5, "mask": {"size": z["window"]},
+           "rot": {"base": 10000.0, "dims": 64}}
+    ssd = {"heads": 2 * w // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}
+    layers = [{"type": "mamba2", "mixer": ssd, "mlp": moe}, {"type": "attention", "mixer": att, "mlp": moe},
+              {"type": "latent_attention", "mixer": lat, "mlp": moe}, {"type": "attention", "mixer": dict(att, kv_from=1), "mlp": moe}]
+    befirax = {"architecture": "Befirax", "vocab": DESIGN_VOCAB, "width": w, "norm": {"eps": 1e-6}, "streams": 2,
+               "layers": [dict(l, mixer=dict(l["mixer"], **({"kv_from": l["mixer"]["kv_from"] + 4 * r} if "kv_from" in l["mixer"] else {})))
+                          for r in range(z["layers"] // 4) for l in layers]}
+    melerax, _, qwen = melerax_configs(z)
+    return befirax, melerax, qwen
+
+
 def compare_designs(args) -> int:
     """Prefill (one prompt in one step) and decode (a batch of single tokens at a context, from the captured step)
     of both designs through the step function; random weights, synthetic tokens.  One JSON line."""
@@ -355,6 +379,8 @@ def compare_designs(args) -> int:
         design = args.design
         if design == "melerax":
             pairs = list(zip(("melerax", "renanex", "qwen2"), melerax_configs(z)))
+        elif design == "befirax":
+            pairs = list(zip(("befirax", "melerax", "qwen2"), befirax_configs(z)))
         else:
             pairs = list(zip((design, "qwen2"), nubodra_configs(z) if design == "nubodra" else design_configs(z)))
         for name, raw in pairs:
@@ -423,9 +449,10 @@ def main() -> int:
     ap.add_argument("--designs", action="store_true",
                     help="instead of the default run: prefill and decode throughput of Renanex layers (Mamba scan, attention whose heads "
                          "exchange scores over a window, lightning attention) beside Qwen2 layers of equal sizes, at a few sizes")
-    ap.add_argument("--design", default="renanex", choices=["renanex", "nubodra", "melerax"],
+    ap.add_argument("--design", default="renanex", choices=["renanex", "nubodra", "melerax", "befirax"],
                     help="with --designs: which design stands beside Qwen2 (nubodra: latent attention and attention behind a convolution, "
-                         "beside Qwen2 layers that see every key; melerax: chunked attention beside a gated linear recurrence, time mixing "
+                         "beside Qwen2 layers that see every key; befirax: state-space duality, differential and latent attention and gated "
+                         "experts over two residual streams, beside Melerax and Qwen2; melerax: chunked attention beside a gated linear recurrence, time mixing "
                          "and routed experts, beside Renanex and Qwen2 layers)")
     ap.add_argument("--design-sizes", default="small,medium", help="with --designs: which of the sizes to run (small, medium, large)")
     ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)

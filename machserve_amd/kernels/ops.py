@@ -1362,10 +1362,16 @@ class HipOps:
         self._want(state, torch.float32, "ssd state", state.shape[0], H, N, P)
         S = self._seq_operands("ssd", seq_q_start, seq_q_len, seq_slot)
         y = torch.empty((T, H * P), dtype=torch.float32, device=xbc.device)
+        seg, n_segs = self._walk_segments(T, S, self.SSD_SEGMENT, H * N * P)
+        carry = torch.empty((S, n_segs, H, N, P), dtype=torch.float32, device=xbc.device) if seg else None
+        cdec = torch.empty((S, n_segs, H), dtype=torch.float32, device=xbc.device) if seg else None
         self._check(lib, lib.ms_ssd_scan(_ptr(xbc), _c_int(xbc.shape[1]), _ptr(proj), _c_int(proj.shape[1]), _c_int(dt_col), _ptr(dt_bias),
                                          _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S),
-                                         _ptr(y), _c_int(T), _c_int(H), _c_int(P), _c_int(N), _c_int(G), self._stream()))
+                                         _ptr(y), _c_int(T), _c_int(H), _c_int(P), _c_int(N), _c_int(G), _c_int(seg), _c_int(n_segs),
+                                         _ptr(carry), _ptr(cdec), self._stream()))
         return y
+
+    SSD_SEGMENT = 64  # rows of a segment of the state-space recurrence
 
     def gated_group_norm(self, y: torch.Tensor, proj: torch.Tensor, z_col: int, weight: torch.Tensor, eps: float, groups: int,
                          out_cols: int) -> torch.Tensor:

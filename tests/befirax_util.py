@@ -7,7 +7,7 @@ import os
 import torch
 
 from plain import befirax_plain as P
-from renanex_util import relative_error, relative_errors, run_schedule, tokens_of, within  # noqa: F401  (shared runners)
+from renanex_util import relative_error, relative_errors, run_schedule, tokens_of  # noqa: F401  (shared runners)
 
 
 def attention(heads, kv, dim, vdim, scale, diff, conv=3, rot=(10000.0, None), kv_from=None):
@@ -124,3 +124,16 @@ def _is_matrix(name: str, t) -> bool:
     if name.endswith((".conv", ".router", ".mix")) or ".hc" in name or t.dim() < 2:
         return False
     return True
+
+
+def within(got: torch.Tensor, want: torch.Tensor, dtype) -> bool:
+    """float32: every row within rounding of sums taken in another order (a key too many or too few, a window one token
+    off or a state that is lost is off by 1e-2 and more).  bfloat16: rounding of activations grows through the layers, so
+    half the rows must be within 4e-2; and where two router scores lie within that rounding of each other a row takes
+    another expert than the plain model does, which moves that row by as much as the expert matters and the rows after it
+    by a little: at most one row in thirty may be beyond 0.25 (logits that have nothing to do with the wanted ones are
+    off by 1.4 in every row)."""
+    e = relative_errors(got, want)
+    if dtype == torch.float32:
+        return float(e.max()) < 1e-4
+    return float(e.median()) < 4e-2 and int((e > 0.25).sum()) <= max(1, e.numel() // 30)
