@@ -109,12 +109,23 @@ __global__ __launch_bounds__(256) void expert_act_kernel(const float* __restrict
     const float* g = gates + (size_t)t * ld_gates;
     if (gated) {  // up [T, 2 n]: the gates' columns, then the up projections'
         const float* row = up + (size_t)t * 2 * n;
+#pragma unroll 2
         for (int c = c0 + threadIdx.x * V; c < c1; c += 256 * V) {
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                const int e = (c + v) / ff;
-                const float w = e < E ? g[e] : 1.0f;
-                out[(size_t)t * n + c + v] = from_f32<elem_t>(w != 0.f ? expert_activation(row[c + v], act) * row[n + c + v] * w : 0.f);
+            const int e = c / ff;  // V columns lie in one expert (ff is a multiple of V)
+            const float w = e < E ? g[e] : 1.0f;
+            elem_t* o = out + (size_t)t * n + c;
+            if constexpr (V == 4) {
+                float4 a = (float4){0.f, 0.f, 0.f, 0.f}, b = a;
+                if (w != 0.f) {
+                    a = *reinterpret_cast<const float4*>(row + c);
+                    b = *reinterpret_cast<const float4*>(row + n + c);
+                }
+                o[0] = from_f32<elem_t>(w != 0.f ? expert_activation(a.x, act) * b.x * w : 0.f);
+                o[1] = from_f32<elem_t>(w != 0.f ? expert_activation(a.y, act) * b.y * w : 0.f);
+                o[2] = from_f32<elem_t>(w != 0.f ? expert_activation(a.z, act) * b.z * w : 0.f);
+                o[3] = from_f32<elem_t>(w != 0.f ? expert_activation(a.w, act) * b.w * w : 0.f);
+            } else {
+                o[0] = from_f32<elem_t>(w != 0.f ? expert_activation(row[c], act) * row[n + c] * w : 0.f);
             }
         }
         return;

@@ -74,16 +74,32 @@ CONFIGS = {
         layer(latent(17, 16, 16, 32, 48, 0.3, base=1000.0, window=200), moe(8, 8, 16, identity=1))], streams=1),
 }
 
+# configurations for the GPU alone (the stand-ins would take minutes): sizes nearer a real model's layers
+MORE_CONFIGS = {
+    # four streams; an attention layer first; heads of 64 with values of 128; a latent of 128 beside a rotated part of 64
+    # and one of 160 beside 32; state-space heads of 64 and 128 with 64 and 128 states; sixteen experts; a layer without
+    # feed-forward in the middle; the reading layer convolves with other taps than the layer it reads
+    "big": model(512, 1000, [
+        layer(attention(8, 2, 64, 128, 0.125, 0.2, conv=2, rot=(10000.0, 64)), moe(16, 4, 128, identity=3)),
+        layer(latent(8, 64, 64, 64, 128, 0.09, base=250000.0, window=64), moe(8, 2, 256)),
+        layer(mamba2(16, 64, 64, 4, 4, 4), moe(16, 4, 128, identity=3)),
+        layer(attention(8, 2, 64, 128, 0.125, 0.35, conv=4, rot=(10000.0, 64), kv_from=0), moe(8, 2, 256)),
+        layer(mamba2(8, 128, 128, 1, 2, 1), None),
+        layer(latent(4, 128, 32, 128, 160, 0.08, base=10000.0), moe(16, 1, 64, identity=1))], streams=4),
+}
+CONFIGS_ALL = dict(CONFIGS, **MORE_CONFIGS)
 
-def make_dir(tmp, name: str, seed: int = 0, sharpen: float = 6.0, dtype=torch.float32) -> str:
+
+def make_dir(tmp, name: str, seed: int = 0, sharpen: float = 6.0, dtype=torch.float32, experts: float = 8.0) -> str:
     """A model folder of random weights, changed so that faults show: embeddings of order one, query and key projections
     times ``sharpen`` (softmaxes far from flat: a key that is missing or one too many shows in the logits), input
     projections of the state-space layers and of the experts of order one, corrections large enough to change the
-    choice, streams that differ from each other."""
+    choice, streams that differ from each other.  ``experts``: the factor on the experts' gate and up projections (large: an
+    expert's output outweighs the stream, and a row whose choice flips under a two-byte type's rounding is lost)."""
     from safetensors.torch import load_file, save_file
     from machserve_amd.weights import write_random_model
-    out = os.path.join(str(tmp), f"befirax_{name}_{seed}")
-    write_random_model(dict(CONFIGS[name]), seed, out, dtype)
+    out = os.path.join(str(tmp), f"befirax_{name}_{seed}_{sharpen}_{experts}")
+    write_random_model(dict(CONFIGS_ALL[name]), seed, out, dtype)
     path = os.path.join(out, "model.safetensors")
     w = load_file(path)
     for k in list(w):
@@ -92,7 +108,9 @@ def make_dir(tmp, name: str, seed: int = 0, sharpen: float = 6.0, dtype=torch.fl
             t = t * 40.0
         elif k.endswith((".mix.q", ".mix.k")):
             t = t * sharpen
-        elif k.endswith((".mix.in", ".mix.v", ".mix.dkv", ".mix.uk", ".mix.uv", ".mix.g", ".up", ".gate")):
+        elif k.endswith((".up", ".gate")):
+            t = t * experts
+        elif k.endswith((".mix.in", ".mix.v", ".mix.dkv", ".mix.uk", ".mix.uv", ".mix.g")):
             t = t * 8.0
         elif k.endswith(".correction"):
             t = t * 10.0
