@@ -4,6 +4,8 @@
 //   read:   u[t] = sum_s w_in[s] xs[s, t]                       (w_in null: the plain sum; of chosen rows if asked)
 //           with a norm: h[t] = u[t] / sqrt(mean(u[t]^2) + eps) * w, in the element type, the same kernel
 //   write:  y[t] = sum_p sums[p, t] + bias;   xs[s', t] <- sum_s mix[s, s'] xs[s, t] + w_out[s'] y[t]   for all s' at once
+//   write and read: a write and the next branch's read with its norm in one kernel (a block a row), which saves the read's
+//           pass over the streams: the new values are summed with the next weights while they are in registers
 //
 // The write kernel adds up the partial sums that a branch's last product left, so that product needs no pass of its own
 // over the streams.  Every thread reads the old values of its columns in all streams before it writes any of them.
@@ -133,6 +135,84 @@ __global__ __launch_bounds__(256) void streams_write_kernel(StreamsWriteArgs a) 
     }
 }
 
+// A write and the next read with its RMS norm: one block a row.  The row of the next branch's input is kept in LDS between
+// the sum of squares and the store; the new values of a column are summed in the order of the streams, as the read
+// kernel sums them, so the result is the same number as from a write and a read.
+struct StreamsWriteReadArgs {
+    StreamsWriteArgs w;
+    const float* w_in;     // [S] of the read that follows, or null: the plain sum
+    const float* norm_w;   // [d]
+    float eps;
+    elem_t* out;           // [T, d]
+};
+
+template <int V>
+__global__ __launch_bounds__(256) void streams_write_read_kernel(StreamsWriteReadArgs q) {
+    const StreamsWriteArgs& a = q.w;
+    __shared__ float m[MAX_STREAMS * MAX_STREAMS + 2 * MAX_STREAMS];
+    __shared__ float scratch[4];
+    extern __shared__ float row[];  // d floats
+    const int SS = a.S * a.S;
+    for (int i = threadIdx.x; i < SS + 2 * a.S; i += 256)
+        m[i] = i < SS ? a.mix[i] : i < SS + a.S ? a.w_out[i - SS] : (q.w_in ? q.w_in[i - SS - a.S] : 1.0f);
+    __syncthreads();
+    const int t = blockIdx.x;
+    const size_t plane = (size_t)a.T * a.d;
+    float ss = 0.f;
+    for (int c = threadIdx.x * V; c < a.d; c += 256 * V) {
+        const size_t at = (size_t)t * a.d + c;
+        float y[V], old[MAX_STREAMS][V], u[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            y[v] = a.bias ? a.bias[c + v] : 0.f;
+            u[v] = 0.f;
+        }
+        for (int p = 0; p < a.P; ++p) {
+            if constexpr (V == 4) {
+                const float4 z = *reinterpret_cast<const float4*>(a.sums + p * plane + at);
+                y[0] += z.x; y[1] += z.y; y[2] += z.z; y[3] += z.w;
+            } else {
+                y[0] += a.sums[p * plane + at];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s) {
+            if (s >= a.S) break;
+            if constexpr (V == 4) {
+                const float4 z = *reinterpret_cast<const float4*>(a.xs + s * plane + at);
+                old[s][0] = z.x; old[s][1] = z.y; old[s][2] = z.z; old[s][3] = z.w;
+            } else {
+                old[s][0] = a.xs[s * plane + at];
+            }
+        }
+#pragma unroll
+        for (int to = 0; to < MAX_STREAMS; ++to) {
+            if (to >= a.S) break;
+            float out[V];
+#pragma unroll
+            for (int v = 0; v < V; ++v) out[v] = m[SS + to] * y[v];
+#pragma unroll
+            for (int s = 0; s < MAX_STREAMS; ++s) {
+                if (s >= a.S) break;
+#pragma unroll
+                for (int v = 0; v < V; ++v) out[v] += m[s * a.S + to] * old[s][v];
+            }
+            if constexpr (V == 4) *reinterpret_cast<float4*>(a.xs + to * plane + at) = (float4){out[0], out[1], out[2], out[3]};
+            else a.xs[to * plane + at] = out[0];
+#pragma unroll
+            for (int v = 0; v < V; ++v) u[v] += m[SS + a.S + to] * out[v];
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            row[c + v] = u[v];
+            ss += u[v] * u[v];
+        }
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)a.d + q.eps);
+    for (int c = threadIdx.x; c < a.d; c += 256) q.out[(size_t)t * a.d + c] = from_f32<elem_t>(row[c] * inv * q.norm_w[c]);
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -167,4 +247,17 @@ extern "C" int ms_streams_write(float* xs, const float* sums, int P, const float
     if (d % 4 == 0) hipLaunchKernelGGL(streams_write_kernel<4>, dim3((unsigned)std::min<long>(ceil_div(n / 4, 256L), 65535L * 16)), dim3(256), 0, stream, a);
     else hipLaunchKernelGGL(streams_write_kernel<1>, dim3((unsigned)std::min<long>(ceil_div(n, 256L), 65535L * 16)), dim3(256), 0, stream, a);
     return check_launch("streams_write");
+}
+
+// The write above and, in the same kernel, the read of the branch that follows: out = rmsnorm(sum_s w_in[s] xs'[s]) * norm_w
+// in the element type, from the streams as they are written.
+extern "C" int ms_streams_write_read(float* xs, const float* sums, int P, const float* bias, const float* mix, const float* w_out,
+                                     const float* w_in, const float* norm_w, float eps, void* out, int S, int T, int d, hipStream_t stream) {
+    MS_REQUIRE(S >= 1 && S <= MAX_STREAMS && T > 0 && d > 0 && P >= 1, "streams_write_read: %d streams (at most %d) of %d rows of %d, %d sums", S,
+               MAX_STREAMS, T, d, P);
+    MS_REQUIRE(d <= STREAMS_MAX_ROW && norm_w && out, "streams_write_read: a normed row of %d numbers (at most %d)", d, STREAMS_MAX_ROW);
+    StreamsWriteReadArgs q{{xs, sums, bias, mix, w_out, P, S, T, d}, w_in, norm_w, eps, (elem_t*)out};
+    if (d % 4 == 0) hipLaunchKernelGGL(streams_write_read_kernel<4>, dim3(T), dim3(256), (size_t)d * sizeof(float), stream, q);
+    else hipLaunchKernelGGL(streams_write_read_kernel<1>, dim3(T), dim3(256), (size_t)d * sizeof(float), stream, q);
+    return check_launch("streams_write_read");
 }

@@ -1341,6 +1341,25 @@ class HipOps:
         self._check(lib, lib.ms_streams_write(_ptr(xs), _ptr(sums), _c_int(sums.shape[0]), _ptr(bias), _ptr(mix), _ptr(w_out), _c_int(S),
                                               _c_int(T), _c_int(d), self._stream()))
 
+    def streams_write_read_norm(self, xs: torch.Tensor, sums: torch.Tensor, bias: Optional[torch.Tensor], mix: torch.Tensor,
+                                w_out: torch.Tensor, w_in: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float) -> torch.Tensor:
+        """:meth:`streams_write` and, from the streams as they are written, :meth:`streams_read_norm` of the branch that
+        follows, in one kernel: the same numbers as the two calls."""
+        lib = self._extra_lib("multistream")
+        S, T, d = self._streams(xs)
+        self._want(sums, torch.float32, "streams' sums", sums.shape[0], T, d)
+        if bias is not None:
+            self._want(bias, torch.float32, "streams' bias", d)
+        self._want(mix, torch.float32, "streams' mixing matrix", S, S)
+        self._want(w_out, torch.float32, "streams' output weights", S)
+        if w_in is not None:
+            self._want(w_in, torch.float32, "streams' input weights", S)
+        self._want(norm_w, torch.float32, "streams' norm weight", d)
+        out = torch.empty((T, d), dtype=self.dtype, device=xs.device)
+        self._check(lib, lib.ms_streams_write_read(_ptr(xs), _ptr(sums), _c_int(sums.shape[0]), _ptr(bias), _ptr(mix), _ptr(w_out), _ptr(w_in),
+                                                   _ptr(norm_w), _c_float(eps), _ptr(out), _c_int(S), _c_int(T), _c_int(d), self._stream()))
+        return out
+
     # ------------------------------------------------------------------ state-space duality
     def ssd_limits(self) -> dict:
         lib = self._extra_lib("ssd")

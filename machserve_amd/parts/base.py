@@ -165,21 +165,38 @@ class ResidualStream:
 class MultiStream:
     """Several 32-bit residual streams ``xs [streams, T, width]``, all equal to the embedding at the start.  A branch reads a
     weighted sum of them and is written back into all of them at once (``parts/block.py``, the multi-stream block); the
-    model's output is their sum."""
+    model's output is their sum.  A write is not launched at once but when the streams are next read: where that
+    reader is a weighted sum under an RMS norm (the next branch's input), one kernel writes and reads."""
 
     def __init__(self, x: torch.Tensor, streams: int, ops):
         self.ops = ops
         self.xs = x.new_empty((streams,) + tuple(x.shape))
         self.xs[:] = x
+        self.pending = None  # (sums, bias, mix, w_out) of a write that has not been launched
+
+    def flush(self) -> None:
+        if self.pending is not None:
+            self.ops.streams_write(self.xs, *self.pending)
+            self.pending = None
 
     def read(self, w_in: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> ResidualStream:
         """``sum_s w_in[s] x_s`` (None: the plain sum), of the ``rows`` if given, as a stream of its own."""
+        self.flush()
         return ResidualStream(self.ops.streams_read(self.xs, w_in, rows), self.ops)
+
+    def read_norm(self, w_in: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float) -> torch.Tensor:
+        """``rmsnorm(sum_s w_in[s] x_s) * norm_w`` in the element type."""
+        if self.pending is not None and hasattr(self.ops, "streams_write_read_norm"):
+            pending, self.pending = self.pending, None
+            return self.ops.streams_write_read_norm(self.xs, *pending, w_in, norm_w, eps)
+        self.flush()
+        return self.ops.streams_read_norm(self.xs, w_in, norm_w, eps)
 
     def write(self, sums: torch.Tensor, bias: Optional[torch.Tensor], mix: torch.Tensor, w_out: torch.Tensor) -> None:
         """All streams at once from the old ones: ``x_t = sum_s mix[s, t] x_s + w_out[t] (sum(sums) + bias)``; ``sums``
         float32 ``[P, T, width]`` are the partial sums of a branch's last product."""
-        self.ops.streams_write(self.xs, sums, bias, mix, w_out)
+        self.flush()
+        self.pending = (sums, bias, mix, w_out)
 
     def value(self) -> torch.Tensor:
         return self.read(None).x

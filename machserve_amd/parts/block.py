@@ -104,7 +104,8 @@ class StreamMix(Part):
 class MultiStreamBlock(Block):
     """Pre-norm over several residual streams (``base.MultiStream``).  Reads ``mixer``, ``feed_forward`` (may be None),
     ``mixer_norm``, ``feed_forward_norm``, ``mixer_streams`` and ``feed_forward_streams`` of its layer's spec.  A branch's
-    input is the norm of ``sum_s in[s] x_s`` (one kernel for the sum and an RMS norm); what it leaves (the operands of a
+    input is the norm of ``sum_s in[s] x_s`` (one kernel for the sum and an RMS norm, which also writes what the branch before
+    left); what it leaves (the operands of a
     last product, a bias, a finished tensor, rows of its input to be added with weights) is written into all streams by
     one kernel that also adds the product's partial sums up."""
 
@@ -135,7 +136,7 @@ class MultiStreamBlock(Block):
     def _branch(self, norm, part, mix, stream, ctx):
         ops = self.rt.ops
         if type(norm).__name__ == "RMSNorm" and hasattr(ops, "streams_read_norm"):
-            h = ops.streams_read_norm(stream.xs, mix.w_in, norm.weight, norm.spec.eps)
+            h = stream.read_norm(mix.w_in, norm.weight, norm.spec.eps)  # one kernel with the write before it, if one is pending
         else:
             h = norm.forward(stream.read(mix.w_in))
         out = _Branch(ops)

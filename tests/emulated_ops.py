@@ -498,6 +498,10 @@ class EmulatedOps:
             y = y + bias
         xs.copy_(torch.einsum("st,snw->tnw", mix, xs) + w_out[:, None, None] * y[None])
 
+    def streams_write_read_norm(self, xs, sums, bias, mix, w_out, w_in, norm_w, eps):
+        self.streams_write(xs, sums, bias, mix, w_out)
+        return self.streams_read_norm(xs, w_in, norm_w, eps)
+
     # ------------------------------------------------------------------ differential attention, state-space duality
     def sigmoid_rows(self, sums):
         return torch.sigmoid(sums)

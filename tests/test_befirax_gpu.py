@@ -76,6 +76,10 @@ def test_streams_read_and_written(dtype, S, d, T):
         got = dev(xs)
         ops.streams_write(got, dev(sums), dev(bias), dev(mix), dev(w_out))
         close(got, want, torch.float32, f"all streams at once from {parts} sums")
+        both = dev(xs)
+        h = ops.streams_write_read_norm(both, dev(sums), dev(bias), dev(mix), dev(w_out), dev(w_in), dev(nw), 1e-5)
+        close(both, want, torch.float32, "a write with the next read in its kernel leaves the same streams")
+        close(h, ref.streams_read_norm(want, w_in, nw, 1e-5), dtype, "and the same input of the next branch")
 
 
 def test_streams_beyond_the_kernels_are_refused():
