@@ -233,20 +233,24 @@ class BefiraxConfig:
             mixer = self._mixer_spec(m, f"l{i}.mix.")
             feed = self._mlp_spec(mlp, f"l{i}.mlp.") if mlp is not None else None
             norm2 = self._norm(f"l{i}.norm2") if mlp is not None else None
+            # a layer without feed-forward uses neither its second norm nor its second streams' tensors, should the
+            # checkpoint have them
+            unused = () if mlp is not None else (f"l{i}.norm2",)
             if self.streams is None:
-                layers.append(LayerSpec("prenorm", mixer, feed, self._norm(f"l{i}.norm1"), norm2))
+                layers.append(LayerSpec("prenorm", mixer, feed, self._norm(f"l{i}.norm1", unused), norm2))
             else:
-                mix = lambda p: StreamMixSpec(self.streams, {"in": p + "in", "out": p + "out", "mix": p + "mix"})
-                layers.append(MultiStreamLayerSpec("multistream", mixer, feed, self._norm(f"l{i}.norm1"), norm2, mix(f"l{i}.hc1."),
-                                                   mix(f"l{i}.hc2.") if mlp is not None else None))
+                mix = lambda p, ignored=(): StreamMixSpec(self.streams, {"in": p + "in", "out": p + "out", "mix": p + "mix"}, ignored=ignored)
+                unused2 = () if mlp is not None else tuple(f"l{i}.hc2.{s}" for s in ("in", "out", "mix"))
+                layers.append(MultiStreamLayerSpec("multistream", mixer, feed, self._norm(f"l{i}.norm1", unused), norm2,
+                                                   mix(f"l{i}.hc1.", unused2), mix(f"l{i}.hc2.") if mlp is not None else None))
         spec = ModelSpec(architecture=ARCHITECTURE, embedding=EmbeddingSpec(self.vocab, self.width, {"weight": "embed"}),
                          layers=tuple(layers), order=tuple(range(len(layers))), final_norm=self._norm("final.norm"),
                          head=HeadSpec(self.vocab, self.width, True), max_positions=MAX_POSITIONS, streams=self.streams)
         spec.validate()
         return spec
 
-    def _norm(self, name: str) -> NormSpec:
-        return NormSpec("rmsnorm", self.width, self.norm_eps, {"weight": name})
+    def _norm(self, name: str, ignored=()) -> NormSpec:
+        return NormSpec("rmsnorm", self.width, self.norm_eps, {"weight": name}, ignored=tuple(ignored))
 
     # ------------------------------------------------------------------ random weights
     def random_tensor_plan(self):

@@ -30,6 +30,8 @@ class NormSpec:
     offset: float = 0.0
     # whether a second vector ("scale" among the tensors) multiplies the normed row as well (a layer's scale)
     scaled: bool = False
+    # checkpoint names that may be present without being used
+    ignored: Sequence[str] = ()
 
 
 @dataclass(frozen=True)
@@ -393,6 +395,8 @@ class StreamMixSpec:
     streams: int
     tensors: Mapping[str, str] = field(default_factory=dict)
     kind: str = "stream_mix"
+    # checkpoint names that may be present without being used
+    ignored: Sequence[str] = ()
 
 
 @dataclass(frozen=True)

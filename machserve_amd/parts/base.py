@@ -258,6 +258,10 @@ class Part:
         """Receive the declared tensors (absent optional ones are None), already on the
         device in the dtype of their role."""
 
+    def ignored_tensors(self) -> List[str]:
+        """Checkpoint names that may be present without being used (a spec may list them as ``ignored``)."""
+        return list(getattr(self.spec, "ignored", ()))
+
 
 class Norm(Part):
     def forward(self, stream: ResidualStream, rows: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -266,3 +266,22 @@ def test_greedy_generation_through_the_scheduler(tmp_path):
     for p, g in zip(prompts, got):
         assert g == P.greedy_generate(w, cfg, p, 5, torch.float64)
     lm.cache.check()
+
+
+def test_a_layer_without_feed_forward_may_bring_its_unused_tensors(tmp_path):
+    """The second norm and the second streams' tensors of a layer that has no feed-forward are not used and not missed;
+    any other tensor the model does not know is still refused by name."""
+    from safetensors.torch import load_file, save_file
+    from machserve_amd.weights.loader import WeightsError
+    d = U.make_dir(tmp_path, "mixed", seed=8)
+    path = d + "/model.safetensors"
+    w = load_file(path)
+    w.update({"l2.norm2": torch.ones(64), "l2.hc2.in": torch.ones(3), "l2.hc2.out": torch.ones(3), "l2.hc2.mix": torch.eye(3)})
+    save_file(w, path)
+    toks = U.tokens_of(9, 97, 1)
+    got = U.run_schedule(loaded(d), {"a": toks}, [[("a", 9)]])["a"]
+    assert U.relative_error(got, U.plain_logits(d, toks)) < TOL
+    w["l2.mlp.router"] = torch.ones(3, 64)
+    save_file(w, path)
+    with pytest.raises(WeightsError, match="l2.mlp.router"):
+        loaded(d)
