@@ -97,11 +97,11 @@ def _mixer_of(kind, m: dict, where: str, index: int):
         src = m.get("kv_from")
         if src is not None and (isinstance(src, bool) or not isinstance(src, int) or not 0 <= src < index):
             raise ConfigError(f"config.json: '{where}kv_from' must name an earlier layer, got {src!r}")
-        diff = _num(m, "diff", where)
-        if diff >= 1.0:
-            raise ConfigError(f"config.json: '{where}diff' must lie below 1, got {diff!r}")
+        diff = _num(m, "diff", where, positive=False)
+        if not 0.0 <= diff < 1.0:
+            raise ConfigError(f"config.json: '{where}diff' must lie in [0, 1), got {diff!r}")
         return DiffAttentionLayer(heads, kv, dim, _int(m, "vdim", where), _num(m, "scale", where), diff,
-                                  _int(m, "conv", where) if m.get("conv") is not None else 0, _rot_of(m, where, dim), src)
+                                  _int(m, "conv", where, 0) if m.get("conv") is not None else 0, _rot_of(m, where, dim), src)
     if kind == "latent_attention":
         rot_dim = _int(m, "rot_dim", where, 2)
         rot = _rot_of(m, where, rot_dim)
